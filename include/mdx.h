@@ -1,0 +1,181 @@
+/*
+ * mdx.h -- C ABI of libmdx.so: the block-diffusion attention hot path of the
+ * nano_dvlm engine (opendatalab/MinerU-Diffusion) as hand-written gfx950 HIP
+ * kernels for one MI355X.
+ *
+ * The reference has no FFI: its hot path is reached through Python call sites.
+ * Each entry point below names the reference interface it stands in for.  All
+ * pointers are BORROWED DEVICE pointers (the caller keeps the memory alive
+ * until the stream has passed the call); outputs and workspaces are allocated
+ * by the caller.  No entry point allocates, frees or synchronises; every
+ * kernel is enqueued on `stream` (a hipStream_t, 0 = the null stream), so all
+ * of them may be recorded into a HIP graph.  The library keeps no global state
+ * apart from a thread-local error string.
+ *
+ * Return value: 0 on success, a negative MDX_E* code otherwise (nothing has
+ * been enqueued then); mdx_last_error() gives the reason as text.
+ */
+#ifndef MDX_H
+#define MDX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MDX_VERSION 100            /* major*10000 + minor*100 + patch */
+
+#define MDX_OK            0
+#define MDX_EINVAL       -1        /* bad argument: null pointer, negative size */
+#define MDX_EUNSUPPORTED -2        /* shape / dtype / stride outside what the kernels cover */
+#define MDX_EWORKSPACE   -3        /* workspace missing or too small */
+#define MDX_ELAUNCH      -4        /* the HIP runtime refused the launch */
+
+#define MDX_BF16 0                 /* element types of q/k/v/o, the caches and the logits */
+#define MDX_F16  1
+#define MDX_F32  2                 /* logits only */
+
+typedef void* mdx_stream_t;        /* hipStream_t */
+
+int         mdx_version(void);
+const char* mdx_last_error(void);  /* thread-local; valid until the next failing call on this thread */
+
+/*
+ * store_kvcache -- replaces store_kvcache / store_kvcache_kernel
+ * (engines/nano_dvlm/nanovllm/layers/attention.py:10-40; 4-D form
+ * layers/sdar_attention.py:11-16 is the same call on flattened views).
+ *
+ * For token i in [0, n_tokens): slot = slot_mapping[i]; if slot == -1 skip,
+ * else copy row_elems elements key + i*k_row_stride -> k_cache + slot*row_elems
+ * and value + i*v_row_stride -> v_cache + slot*row_elems.  Strides are in
+ * elements; rows themselves are dense (attention.py:36-38).  elem_size is in
+ * bytes (2 for bf16/f16).  Slots outside [0, num_slots) are skipped instead
+ * of written (the reference leaves them undefined); num_slots = pages*page.
+ * If two tokens name the same slot the result holds one of the two rows.
+ */
+int mdx_store_kvcache(const void* key, const void* value,
+                      int64_t k_row_stride, int64_t v_row_stride,
+                      void* k_cache, void* v_cache,
+                      const int32_t* slot_mapping,
+                      int64_t n_tokens, int64_t row_elems, int32_t elem_size,
+                      int64_t num_slots, mdx_stream_t stream);
+
+/*
+ * Staircase block-prefill attention over packed variable-length sequences --
+ * replaces sparse_attn_varlen / sparse_attn_varlen_v2
+ * (engines/nano_dvlm/nanovllm/kernels/triton/attention/block_prefill_attention_v2.py:16-202).
+ *
+ * q,o [total_tokens, Hq, d]; k,v [total_tokens, Hkv, d]; the innermost stride
+ * is 1, token and head strides are given in elements (so the strided views of
+ * a fused QKV projection are read in place; the reference copies them,
+ * :182).  cu_seqlens_q / cu_seqlens_k [batch+1] int32 device arrays; the
+ * kernel is a self-attention and reads the sequence bounds from cu_seqlens_k,
+ * like the reference (:48-50); both must describe the same sequences.
+ * Blocks of staircase_size tokens (1,2,..,128) are right-aligned in every
+ * sequence (:52-53, :98-102): query i sees key j iff
+ * j <= ((i+pad)/S+1)*S-1-pad, pad = ceil(L/S)*S-L.  Hq % Hkv == 0 and
+ * kv head = q head / (Hq/Hkv) (:34).  softmax(q k^T * scale) v with fp32
+ * accumulation.  max_seqlen is an upper bound on the longest sequence (it
+ * sizes the grid; total_tokens is always a valid bound).  Supported: d == 128,
+ * dtype MDX_BF16.
+ */
+int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
+                              int64_t q_stride_t, int64_t q_stride_h,
+                              int64_t k_stride_t, int64_t k_stride_h,
+                              int64_t v_stride_t, int64_t v_stride_h,
+                              int64_t o_stride_t, int64_t o_stride_h,
+                              const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                              int32_t batch, int32_t max_seqlen, int64_t total_tokens,
+                              int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                              int32_t staircase_size, float scale, int32_t dtype,
+                              mdx_stream_t stream);
+
+/*
+ * Paged single-block ("decode") attention -- replaces the call
+ * flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=, block_table=,
+ * softmax_scale=, causal=False) of
+ * engines/nano_dvlm/nanovllm/layers/sdar_attention.py:48-56 (flash-attn 2.8.3,
+ * third party; inputs built by engine/model_runner.py:121-125,169-185).
+ *
+ * q,o [bs, Sq, Hq, d] with strides (q_stride_b, q_stride_s, q_stride_h, 1);
+ * caches [num_pages, page_size, Hkv, d] with strides (cache_stride_page,
+ * cache_stride_tok, cache_stride_head, 1); block_table [bs, max_pages] int32,
+ * row stride bt_stride, entries past ceil(ctx/page_size) are not read (-1
+ * padding, model_runner.py:123); context_lens [bs] int32.  Every query of
+ * sequence b sees keys 0..context_lens[b]-1 (non-causal).  Rows with
+ * context_lens[b] == 0 (graph padding, model_runner.py:205-208) produce
+ * zeros.  Page ids outside [0, num_pages) are treated as holding no keys.
+ * The workspace holds the split-KV partial results; its size comes from
+ * mdx_paged_block_attn_workspace_bytes with the same shape arguments.
+ * Supported: d == 128, Sq*(Hq/Hkv) <= 64, page_size % 32 == 0, MDX_BF16.
+ */
+int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
+                                             int32_t num_kv_heads, int32_t head_dim,
+                                             int32_t max_pages, int32_t page_size);
+int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void* v_cache,
+                         int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                         int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                         int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                         const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                         int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                         int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                         float scale, int32_t dtype,
+                         void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+
+/*
+ * Confidence + argmax over the vocabulary -- replaces Sampler.prepare
+ * (engines/nano_dvlm/nanovllm/layers/sampler.py:11-22).
+ *
+ * logits [rows, vocab] (row stride in elements, dtype MDX_BF16/F16/F32);
+ * temperatures: one float per group of rows_per_temp consecutive rows
+ * ([bs] with rows_per_temp = block length; sampler.py:13), or NULL for 1.0;
+ * noise: optional [rows, vocab] fp32 added to logits/T before the argmax
+ * (the Gumbel term of sampler.py:15-18, made an explicit input so the kernel
+ * holds no RNG), or NULL for the plain argmax.  Outputs: x0[r] = first index
+ * of the maximum (int64), x0_p[r] = softmax(logits/T)[x0[r]] (fp32).
+ * Workspace from mdx_confidence_argmax_workspace_bytes (may be 0 bytes: then
+ * workspace may be NULL).
+ */
+int64_t mdx_confidence_argmax_workspace_bytes(int64_t rows, int64_t vocab);
+int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
+                          const float* temperatures, int32_t rows_per_temp,
+                          const float* noise, int64_t noise_row_stride,
+                          int64_t* x0, float* x0_p,
+                          int64_t rows, int64_t vocab,
+                          void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+
+/*
+ * Selection of the positions to commit -- replaces the CPU loop of
+ * Sampler.forward (layers/sampler.py:32-54) and _select_transfer_index
+ * (mineru_diffusion/modeling_mineru_diffusion.py:518-532) on the device.
+ *
+ * Per sequence b (block length S <= 1024): masked = tokens[b,:] == mask_token_id;
+ * conf = masked ? x0_p : -inf; hi = conf > threshold (strict).  If
+ * count(hi) >= k commit all of hi, else commit the min(k, count(masked)) most
+ * confident masked positions (ties: lower position first).  k = 1 gives the
+ * engine's rule (sampler.py:41-50), k = block/steps the HF rule.  Writes
+ * transfer[b,p] (uint8 0/1), tokens[b,p] = x0[b,p] where committed (in place),
+ * and count[b] = number committed (int32).
+ */
+int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t* tokens,
+                        int64_t mask_token_id, float threshold, int32_t k,
+                        uint8_t* transfer, int32_t* count,
+                        int32_t bs, int32_t block_len, mdx_stream_t stream);
+
+/*
+ * The whole unmask step: mdx_confidence_argmax over [bs*block_len, vocab]
+ * followed by mdx_select_transfer, on one stream (sampler.py:24-61 without
+ * the host round trip).  temperatures [bs] or NULL.
+ */
+int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
+                    const float* temperatures, const float* noise, int64_t noise_row_stride,
+                    int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                    int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                    int32_t bs, int32_t block_len, int64_t vocab,
+                    void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MDX_H */

@@ -1,0 +1,202 @@
+// Staircase block-prefill attention over packed variable-length sequences.
+//
+// Query row i of a sequence of length L sees key j iff
+//   j <= ((i + pad) / S + 1) * S - 1 - pad,   pad = ceil(L/S)*S - L
+// (blocks of S tokens, right-aligned; semantics of
+// engines/nano_dvlm/nanovllm/kernels/triton/attention/block_prefill_attention_v2.py:46-53,82-102,134-156).
+//
+// Work decomposition (not the reference's one-program-per-(sequence, head)):
+// everything is indexed in PADDED coordinates ip = i + pad, jp = j + pad, in
+// which block boundaries fall on multiples of S.  A workgroup of 4 wavefronts
+// owns 128 consecutive padded query rows of one sequence and one group of NH
+// query heads sharing a KV head; wavefront w owns rows 32w..32w+31.  For
+// S >= 32 every 32-row tile lies inside one block, so all its rows share one
+// key limit and no element of the tile interior is ever masked: only the very
+// first keys (jp < pad) and, for S < 32, the tiles straddling the limit take
+// the masked path.  K/V tiles of 64 keys are staged once per workgroup in LDS
+// (global -> registers one tile ahead -> LDS) and reused by all 4 wavefronts
+// and by the NH heads of the GQA group.
+//
+// Launch order: workgroups are numbered heaviest-first (last row group of every
+// sequence first), and the head group is the fastest-varying index so that
+// consecutive workgroups, which the dispatcher deals round-robin to the 8 XCDs,
+// keep one KV head's K/V stream per XCD L2 when there are 8 head groups.
+#include "mdx_common.h"
+#include "attn_tile.h"
+
+namespace {
+
+using namespace mdx_attn;
+
+constexpr int kTileKeys = 64;      // keys staged in LDS per iteration
+constexpr int kRowsPerWg = 128;    // 4 wavefronts x 32 query rows
+
+struct StaircaseParams {
+    const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o;
+    int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;   // element strides: token, head
+    const int32_t* cu_seqlens;
+    int batch, n_row_groups, n_head_groups, heads_per_kv;      // heads_per_kv = Hq / Hkv
+    int log2_s;
+    float c;                                                   // scale * log2(e)
+};
+
+template <int NH>
+__global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const StaircaseParams P)
+{
+    __shared__ __attribute__((aligned(16))) char lds_k[kTileKeys * kLdsPitch];
+    __shared__ __attribute__((aligned(16))) char lds_v[kTileKeys * kLdsPitch];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int H = lane >> 5, r = lane & 31;
+
+    // workgroup -> (head group, sequence, row group), heaviest row groups first
+    int id = blockIdx.x;
+    const int hg = id % P.n_head_groups; id /= P.n_head_groups;
+    const int b = id % P.batch;          id /= P.batch;
+    const int rg = P.n_row_groups - 1 - id;
+
+    const int seq0 = P.cu_seqlens[b];
+    const int L = P.cu_seqlens[b + 1] - seq0;
+    if (L <= 0) return;
+    const int S = 1 << P.log2_s;
+    const int Lp = ((L + S - 1) >> P.log2_s) << P.log2_s;     // padded length
+    const int pad = Lp - L;
+    const int row_g0 = rg * kRowsPerWg;                        // first padded row of the workgroup
+    if (row_g0 >= Lp) return;
+
+    const int head0 = hg * NH;
+    const int kvh = head0 / P.heads_per_kv;
+
+    // ---- this wavefront's 32 rows ----
+    const int row_w0 = row_g0 + wave * 32;
+    const int ip = row_w0 + r;                                 // this lane's padded query row
+    const bool row_ok = ip >= pad && ip < Lp;
+    const int64_t tok = (int64_t)seq0 + (ip - pad);
+    bf16x8 q[NH][8];
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+        load_q(q[h], row_ok ? P.q + tok * P.q_st + (int64_t)(head0 + h) * P.q_sh : nullptr, H);
+
+    // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
+    auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
+    const int key_hi = limit_of(ip);
+    const int wave_hi = (row_w0 < Lp) ? limit_of(min(row_w0 + 31, Lp - 1)) : 0;   // 0: idle wavefront
+    const int wave_hi_min = limit_of(row_w0);
+    const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
+    const int n_tiles = (wg_hi + kTileKeys - 1) / kTileKeys;
+
+    WaveState<NH> st;
+    st.init();
+
+    // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t ----
+    const __bf16* kbase = P.k + (int64_t)kvh * P.k_sh;
+    const __bf16* vbase = P.v + (int64_t)kvh * P.v_sh;
+    const int chunk = tid & 15, trow = tid >> 4;
+    TileRegs<kTileKeys> regs;
+    auto fetch = [&](int t) {
+#pragma unroll
+        for (int p = 0; p < kTileKeys / 16; ++p) {
+            const int jp = t * kTileKeys + trow + 16 * p;
+            const bool ok = jp >= pad && jp < Lp;
+            if (ok) {
+                const int64_t kt = (int64_t)seq0 + (jp - pad);
+                regs.k[p] = *reinterpret_cast<const u32x4*>(kbase + kt * P.k_st + chunk * 8);
+                regs.v[p] = *reinterpret_cast<const u32x4*>(vbase + kt * P.v_st + chunk * 8);
+            } else {
+                regs.k[p] = u32x4{0, 0, 0, 0};
+                regs.v[p] = u32x4{0, 0, 0, 0};
+            }
+        }
+    };
+
+    fetch(0);
+    for (int t = 0; t < n_tiles; ++t) {
+        __syncthreads();                       // everyone is done reading the previous tile
+        store_tile<kTileKeys>(lds_k, lds_v, regs, tid);
+        __syncthreads();
+        if (t + 1 < n_tiles) fetch(t + 1);     // in flight while this tile is consumed
+
+        const int key0 = t * kTileKeys;
+        if (key0 < wave_hi) {
+            const bool full = key0 >= pad && key0 + kTileKeys <= wave_hi_min;
+            if (full) {
+                attn_step<NH, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+            } else if (key0 + 32 < wave_hi) {
+                attn_step<NH, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+            } else {
+                attn_step<NH, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+            }
+        }
+    }
+
+    // ---- epilogue: O = O^T / l, bf16, 4 consecutive d per store ----
+    if (!row_ok) return;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+        const float inv = 1.0f / both_halves_sum(st.l[h]);
+        __bf16* orow = P.o + tok * P.o_st + (int64_t)(head0 + h) * P.o_sh;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+                bf16x4 out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[h][dt][4 * g + e] * inv);
+                *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+            }
+    }
+}
+
+}  // namespace
+
+extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
+                                         int64_t q_stride_t, int64_t q_stride_h,
+                                         int64_t k_stride_t, int64_t k_stride_h,
+                                         int64_t v_stride_t, int64_t v_stride_h,
+                                         int64_t o_stride_t, int64_t o_stride_h,
+                                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                                         int32_t batch, int32_t max_seqlen, int64_t total_tokens,
+                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                         int32_t staircase_size, float scale, int32_t dtype,
+                                         mdx_stream_t stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MDX_REQUIRE(batch >= 0 && total_tokens >= 0 && max_seqlen >= 0, MDX_EINVAL, "staircase_attn: negative size");
+    MDX_REQUIRE(dtype == MDX_BF16, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (only bf16)", dtype);
+    MDX_REQUIRE(head_dim == kHeadDim, MDX_EUNSUPPORTED, "staircase_attn: head_dim %d (only 128)", head_dim);
+    MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
+                "staircase_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
+    int log2_s = -1;
+    for (int i = 0; i <= 7; ++i) if (staircase_size == (1 << i)) log2_s = i;
+    MDX_REQUIRE(log2_s >= 0, MDX_EINVAL, "staircase_attn: staircase_size %d not in {1,2,...,128}", staircase_size);
+    MDX_REQUIRE(scale > 0.f, MDX_EINVAL, "staircase_attn: scale must be positive");
+    if (batch == 0 || total_tokens == 0 || max_seqlen == 0) return MDX_OK;
+    MDX_REQUIRE(q && k && v && o && cu_seqlens_q && cu_seqlens_k, MDX_EINVAL, "staircase_attn: null pointer");
+    MDX_REQUIRE(total_tokens < ((int64_t)1 << 31) - 256, MDX_EUNSUPPORTED, "staircase_attn: too many tokens");
+    // 16-byte vector access to every row of q/k/v, 8-byte to o
+    MDX_REQUIRE(mdx::aligned16(q) && mdx::aligned16(k) && mdx::aligned16(v) && mdx::aligned16(o) &&
+                q_stride_t % 8 == 0 && q_stride_h % 8 == 0 && k_stride_t % 8 == 0 && k_stride_h % 8 == 0 &&
+                v_stride_t % 8 == 0 && v_stride_h % 8 == 0 && o_stride_t % 4 == 0 && o_stride_h % 4 == 0,
+                MDX_EUNSUPPORTED, "staircase_attn: q/k/v/o must be 16-byte aligned with strides that are multiples of 8 elements");
+
+    const int G = num_q_heads / num_kv_heads;
+    const int NH = (G % 2 == 0) ? 2 : 1;
+    StaircaseParams P;
+    P.q = (const __bf16*)q; P.k = (const __bf16*)k; P.v = (const __bf16*)v; P.o = (__bf16*)o;
+    P.q_st = q_stride_t; P.q_sh = q_stride_h; P.k_st = k_stride_t; P.k_sh = k_stride_h;
+    P.v_st = v_stride_t; P.v_sh = v_stride_h; P.o_st = o_stride_t; P.o_sh = o_stride_h;
+    P.cu_seqlens = cu_seqlens_k;
+    P.batch = batch;
+    const int64_t max_l = max_seqlen < total_tokens ? max_seqlen : total_tokens;
+    P.n_row_groups = (int)((max_l + staircase_size - 1 + kRowsPerWg - 1) / kRowsPerWg);
+    P.n_head_groups = num_q_heads / NH;
+    P.heads_per_kv = G;
+    P.log2_s = log2_s;
+    P.c = scale * kLog2e;
+    const int64_t grid = (int64_t)P.n_row_groups * batch * P.n_head_groups;
+    MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
+    if (NH == 2) staircase_attn_kernel<2><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    else         staircase_attn_kernel<1><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    return mdx::check_launch("staircase_attn");
+}

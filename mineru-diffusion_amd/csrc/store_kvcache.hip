@@ -1,0 +1,151 @@
+// store_kvcache: scatter of K/V rows into the paged cache.
+//
+// Pure HBM-bound copy (read 2 rows, write 2 rows per token), so there is no
+// MFMA here: every lane moves 16 bytes, a token's K row and V row are each
+// read as one fully coalesced stream, and each workgroup keeps several tokens'
+// loads in flight before the first store is issued.
+//
+// Semantics follow engines/nano_dvlm/nanovllm/layers/attention.py:10-40.
+#include "mdx_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTokPerWg = 4;       // tokens whose loads one workgroup keeps in flight
+
+// Fast path: rows are multiples of 16 B, all bases and strides 16-B aligned,
+// and one token's K+V chunks (2*row16) fit one pass of the workgroup.
+// Chunk c < row16 is K, c >= row16 is V.
+__global__ __launch_bounds__(kThreads) void store_kvcache_vec16(
+    const u32x4* __restrict__ key, const u32x4* __restrict__ value,
+    int64_t k_stride16, int64_t v_stride16,
+    u32x4* __restrict__ k_cache, u32x4* __restrict__ v_cache,
+    const int32_t* __restrict__ slot_mapping,
+    int64_t n_tokens, int row16, int64_t num_slots)
+{
+    const int c = threadIdx.x;
+    const bool is_v = c >= row16;
+    const int cc = is_v ? c - row16 : c;
+    const bool lane_on = c < 2 * row16;
+    const int64_t tok0 = (int64_t)blockIdx.x * kTokPerWg;
+
+    u32x4 buf[kTokPerWg];
+    int64_t slot[kTokPerWg];
+#pragma unroll
+    for (int t = 0; t < kTokPerWg; ++t) {
+        const int64_t tok = tok0 + t;
+        slot[t] = -1;
+        if (tok < n_tokens) {
+            const int64_t s = slot_mapping[tok];
+            if (s >= 0 && s < num_slots) slot[t] = s;
+        }
+        if (slot[t] >= 0 && lane_on) {
+            const u32x4* src = is_v ? value + tok * v_stride16 : key + tok * k_stride16;
+            buf[t] = __builtin_nontemporal_load(src + cc);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kTokPerWg; ++t) {
+        if (slot[t] >= 0 && lane_on) {
+            u32x4* dst = (is_v ? v_cache : k_cache) + slot[t] * row16;
+            dst[cc] = buf[t];
+        }
+    }
+}
+
+// Same, for rows longer than one pass of the workgroup.
+__global__ __launch_bounds__(kThreads) void store_kvcache_vec16_long(
+    const u32x4* __restrict__ key, const u32x4* __restrict__ value,
+    int64_t k_stride16, int64_t v_stride16,
+    u32x4* __restrict__ k_cache, u32x4* __restrict__ v_cache,
+    const int32_t* __restrict__ slot_mapping,
+    int64_t n_tokens, int row16, int64_t num_slots)
+{
+    const int64_t tok = blockIdx.x;
+    if (tok >= n_tokens) return;
+    const int64_t s = slot_mapping[tok];
+    if (s < 0 || s >= num_slots) return;
+    const u32x4* ks = key + tok * k_stride16;
+    const u32x4* vs = value + tok * v_stride16;
+    u32x4* kd = k_cache + s * row16;
+    u32x4* vd = v_cache + s * row16;
+    for (int c = threadIdx.x; c < row16; c += kThreads) {
+        const u32x4 a = __builtin_nontemporal_load(ks + c);
+        const u32x4 b = __builtin_nontemporal_load(vs + c);
+        kd[c] = a;
+        vd[c] = b;
+    }
+}
+
+// Fallback for unaligned bases/strides or odd row sizes: element-wise copy.
+template <typename E>
+__global__ __launch_bounds__(kThreads) void store_kvcache_elem(
+    const E* __restrict__ key, const E* __restrict__ value,
+    int64_t k_stride, int64_t v_stride,
+    E* __restrict__ k_cache, E* __restrict__ v_cache,
+    const int32_t* __restrict__ slot_mapping,
+    int64_t n_tokens, int64_t row_elems, int64_t num_slots)
+{
+    const int64_t tok = blockIdx.x;
+    if (tok >= n_tokens) return;
+    const int64_t s = slot_mapping[tok];
+    if (s < 0 || s >= num_slots) return;
+    for (int64_t c = threadIdx.x; c < row_elems; c += kThreads) {
+        k_cache[s * row_elems + c] = key[tok * k_stride + c];
+        v_cache[s * row_elems + c] = value[tok * v_stride + c];
+    }
+}
+
+}  // namespace
+
+extern "C" int mdx_store_kvcache(const void* key, const void* value,
+                                 int64_t k_row_stride, int64_t v_row_stride,
+                                 void* k_cache, void* v_cache,
+                                 const int32_t* slot_mapping,
+                                 int64_t n_tokens, int64_t row_elems, int32_t elem_size,
+                                 int64_t num_slots, mdx_stream_t stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MDX_REQUIRE(n_tokens >= 0 && row_elems > 0 && num_slots >= 0, MDX_EINVAL,
+                "store_kvcache: negative size (n_tokens=%lld row_elems=%lld num_slots=%lld)",
+                (long long)n_tokens, (long long)row_elems, (long long)num_slots);
+    MDX_REQUIRE(elem_size == 1 || elem_size == 2 || elem_size == 4 || elem_size == 8, MDX_EUNSUPPORTED,
+                "store_kvcache: elem_size %d not in {1,2,4,8}", elem_size);
+    if (n_tokens == 0) return MDX_OK;
+    MDX_REQUIRE(key && value && k_cache && v_cache && slot_mapping, MDX_EINVAL, "store_kvcache: null pointer");
+    MDX_REQUIRE(n_tokens < (int64_t)1 << 31, MDX_EUNSUPPORTED, "store_kvcache: n_tokens %lld too large", (long long)n_tokens);
+    // key.stride(0) may be anything >= 0 for a broadcast, but rows are dense (attention.py:36-37).
+    MDX_REQUIRE(k_row_stride >= 0 && v_row_stride >= 0, MDX_EUNSUPPORTED, "store_kvcache: negative row stride");
+
+    const int64_t row_bytes = row_elems * elem_size;
+    const bool vec_ok = row_bytes % 16 == 0 && (k_row_stride * elem_size) % 16 == 0 &&
+                        (v_row_stride * elem_size) % 16 == 0 && mdx::aligned16(key) && mdx::aligned16(value) &&
+                        mdx::aligned16(k_cache) && mdx::aligned16(v_cache) && row_bytes / 16 < (1 << 30);
+    if (vec_ok) {
+        const int row16 = (int)(row_bytes / 16);
+        const int64_t ks16 = k_row_stride * elem_size / 16, vs16 = v_row_stride * elem_size / 16;
+        if (2 * row16 <= kThreads) {
+            const unsigned grid = (unsigned)((n_tokens + kTokPerWg - 1) / kTokPerWg);
+            store_kvcache_vec16<<<grid, kThreads, 0, stream>>>(
+                (const u32x4*)key, (const u32x4*)value, ks16, vs16, (u32x4*)k_cache, (u32x4*)v_cache,
+                slot_mapping, n_tokens, row16, num_slots);
+        } else {
+            store_kvcache_vec16_long<<<(unsigned)n_tokens, kThreads, 0, stream>>>(
+                (const u32x4*)key, (const u32x4*)value, ks16, vs16, (u32x4*)k_cache, (u32x4*)v_cache,
+                slot_mapping, n_tokens, row16, num_slots);
+        }
+    } else {
+#define MDX_STORE_ELEM(E)                                                                         \
+        store_kvcache_elem<E><<<(unsigned)n_tokens, kThreads, 0, stream>>>(                       \
+            (const E*)key, (const E*)value, k_row_stride, v_row_stride, (E*)k_cache, (E*)v_cache, \
+            slot_mapping, n_tokens, row_elems, num_slots)
+        switch (elem_size) {
+            case 1: MDX_STORE_ELEM(uint8_t); break;
+            case 2: MDX_STORE_ELEM(uint16_t); break;
+            case 4: MDX_STORE_ELEM(uint32_t); break;
+            default: MDX_STORE_ELEM(uint64_t); break;
+        }
+#undef MDX_STORE_ELEM
+    }
+    return mdx::check_launch("store_kvcache");
+}

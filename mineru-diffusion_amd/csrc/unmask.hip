@@ -1,0 +1,425 @@
+// The per-block confidence unmask step: softmax confidence + first-index argmax
+// over the vocabulary, then threshold / top-k selection of masked positions.
+//
+// The vocabulary pass is a single HBM stream over the logits (311 MB at
+// [32 x 32 x 151936] bf16), so it is built for bandwidth, not MFMA: 16-byte
+// coalesced loads, several in flight per lane, an online (max, sum-of-exp)
+// pair per lane that is only rescaled when a 16-byte chunk raises the running
+// maximum, wavefront shuffles and one LDS hop for the row reduction.  The
+// argmax is found without per-element index bookkeeping: a lane remembers the
+// first chunk that set its maximum and re-reads that one chunk at the end.
+//
+// Semantics follow engines/nano_dvlm/nanovllm/layers/sampler.py:11-61 and
+// mineru_diffusion/modeling_mineru_diffusion.py:518-532.
+#include "mdx_common.h"
+#include <hip/hip_fp16.h>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;               // 16-byte loads in flight per lane
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegBig = -3.0e38f;      // finite stand-in for -inf: keeps (m - m) away from inf - inf
+constexpr int kNoIndex = 0x7fffffff;
+
+struct Partial {                         // one row's (or row split's) running state
+    float m;                             // max of the raw logits seen
+    float s;                             // sum of exp((x - m)/T)
+    int idx;                             // first index holding m
+    float pick;                          // with noise: best (x/T + g); else unused
+    float pick_x;                        // with noise: raw logit at that index
+    int pick_idx;                        // with noise: first index of the best
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Combine b into a.  c = log2(e)/T.
+__device__ __forceinline__ void combine(Partial& a, const Partial& b, float c, bool noise) {
+    const float M = fmaxf(a.m, b.m);
+    a.s = a.s * fast_exp2((a.m - M) * c) + b.s * fast_exp2((b.m - M) * c);
+    a.idx = (b.m > a.m) ? b.idx : ((b.m == a.m) ? min(a.idx, b.idx) : a.idx);
+    a.m = M;
+    if (noise) {
+        const bool take = (b.pick > a.pick) || (b.pick == a.pick && b.pick_idx < a.pick_idx);
+        if (take) { a.pick = b.pick; a.pick_x = b.pick_x; a.pick_idx = b.pick_idx; }
+    }
+}
+
+__device__ __forceinline__ Partial shfl_xor(const Partial& p, int mask, bool noise) {
+    Partial r;
+    r.m = __shfl_xor(p.m, mask);
+    r.s = __shfl_xor(p.s, mask);
+    r.idx = __shfl_xor(p.idx, mask);
+    if (noise) {
+        r.pick = __shfl_xor(p.pick, mask);
+        r.pick_x = __shfl_xor(p.pick_x, mask);
+        r.pick_idx = __shfl_xor(p.pick_idx, mask);
+    } else {
+        r.pick = kNegBig; r.pick_x = 0.f; r.pick_idx = kNoIndex;
+    }
+    return r;
+}
+
+// --- element access by logits type: EPC = elements per 16-byte chunk ---------
+template <typename T> struct Elem;
+template <> struct Elem<__bf16> {
+    static constexpr int EPC = 8;
+    static __device__ __forceinline__ void unpack(const u32x4& u, float* x) {
+        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            x[2 * i] = __uint_as_float(w[i] << 16);
+            x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ float one(const __bf16* p) {
+        return __uint_as_float((uint32_t)(*reinterpret_cast<const uint16_t*>(p)) << 16);
+    }
+};
+template <> struct Elem<__half> {
+    static constexpr int EPC = 8;
+    static __device__ __forceinline__ void unpack(const u32x4& u, float* x) {
+        const __half2* h = reinterpret_cast<const __half2*>(&u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float2 f = __half22float2(h[i]);
+            x[2 * i] = f.x;
+            x[2 * i + 1] = f.y;
+        }
+    }
+    static __device__ __forceinline__ float one(const __half* p) { return __half2float(*p); }
+};
+template <> struct Elem<float> {
+    static constexpr int EPC = 4;
+    static __device__ __forceinline__ void unpack(const u32x4& u, float* x) {
+        x[0] = __uint_as_float(u.x); x[1] = __uint_as_float(u.y);
+        x[2] = __uint_as_float(u.z); x[3] = __uint_as_float(u.w);
+    }
+    static __device__ __forceinline__ float one(const float* p) { return *p; }
+};
+
+// One element through the slow path (row head/tail, and every element when a
+// noise tensor is given).  With noise, l = x / T is a true fp32 division so the
+// noisy argmax matches an fp32 host computation bit for bit.
+template <bool NOISE>
+__device__ __forceinline__ void visit(Partial& p, float x, int index, float c, float T, float g) {
+    if (x > p.m) {
+        p.s *= fast_exp2((p.m - x) * c);
+        p.m = x;
+        p.idx = index;
+    } else if (x == p.m && index < p.idx) {
+        p.idx = index;
+    }
+    p.s += fast_exp2((x - p.m) * c);
+    if (NOISE) {
+        const float l = x / T;
+        const float v = l + g;
+        if (v > p.pick || (v == p.pick && index < p.pick_idx)) { p.pick = v; p.pick_x = x; p.pick_idx = index; }
+    }
+}
+
+// grid = (rows, nsplit).  Each workgroup reduces chunks [split*cps, (split+1)*cps)
+// of one row; split 0 also takes the unaligned head and tail elements.
+template <typename T, bool NOISE>
+__global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
+    const T* __restrict__ logits, int64_t row_stride,
+    const float* __restrict__ temperatures, int rows_per_temp,
+    const float* __restrict__ noise, int64_t noise_row_stride,
+    int64_t vocab, int nsplit,
+    Partial* __restrict__ partials,          // [rows, nsplit] when nsplit > 1
+    int64_t* __restrict__ x0, float* __restrict__ x0_p)
+{
+    constexpr int EPC = Elem<T>::EPC;
+    const int64_t row = blockIdx.x;
+    const int split = blockIdx.y;
+    const int tid = threadIdx.x;
+    const T* rp = logits + row * row_stride;
+    const float* np = NOISE ? noise + row * noise_row_stride : nullptr;
+    const float T_ = temperatures ? temperatures[row / rows_per_temp] : 1.0f;
+    const float c = kLog2e / T_;
+
+    // Row geometry: `lead` scalar elements up to the first 16-byte boundary,
+    // `nchunk` aligned chunks, then a scalar tail.
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(rp);
+    int64_t lead = ((16 - (addr & 15)) & 15) / sizeof(T);
+    if (lead > vocab) lead = vocab;
+    const int64_t nchunk = (vocab - lead) / EPC;
+    const int64_t tail0 = lead + nchunk * EPC;
+    const u32x4* cp = reinterpret_cast<const u32x4*>(rp + lead);
+
+    const int64_t cps = (nchunk + nsplit - 1) / nsplit;      // chunks per split
+    const int64_t cbeg = split * cps;
+    const int64_t cend = min(nchunk, cbeg + cps);
+
+    Partial p;
+    p.m = kNegBig; p.s = 0.f; p.idx = kNoIndex; p.pick = kNegBig; p.pick_x = 0.f; p.pick_idx = kNoIndex;
+
+    if (!NOISE) {
+        float m = kNegBig, s = 0.f;
+        int64_t first_chunk = -1;
+        int64_t ch = cbeg + tid;
+        // Main loop: kUnroll loads in flight, then reduce them in order.
+        for (; ch + (int64_t)(kUnroll - 1) * kThreads < cend; ch += (int64_t)kUnroll * kThreads) {
+            u32x4 u[kUnroll];
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) u[k] = __builtin_nontemporal_load(cp + ch + (int64_t)k * kThreads);
+#pragma unroll
+            for (int k = 0; k < kUnroll; ++k) {
+                float x[EPC];
+                Elem<T>::unpack(u[k], x);
+                float cm = x[0];
+#pragma unroll
+                for (int i = 1; i < EPC; ++i) cm = fmaxf(cm, x[i]);
+                if (cm > m) {
+                    first_chunk = ch + (int64_t)k * kThreads;
+                    s *= fast_exp2((m - cm) * c);
+                    m = cm;
+                }
+                const float mc = -m * c;
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) acc += fast_exp2(fmaf(x[i], c, mc));
+                s += acc;
+            }
+        }
+        for (; ch < cend; ch += kThreads) {
+            const u32x4 u = __builtin_nontemporal_load(cp + ch);
+            float x[EPC];
+            Elem<T>::unpack(u, x);
+            float cm = x[0];
+#pragma unroll
+            for (int i = 1; i < EPC; ++i) cm = fmaxf(cm, x[i]);
+            if (cm > m) {
+                first_chunk = ch;
+                s *= fast_exp2((m - cm) * c);
+                m = cm;
+            }
+            const float mc = -m * c;
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < EPC; ++i) acc += fast_exp2(fmaf(x[i], c, mc));
+            s += acc;
+        }
+        p.m = m;
+        p.s = s;
+        if (first_chunk >= 0) {      // locate the first element of that chunk equal to the lane's maximum
+            const u32x4 u = cp[first_chunk];
+            float x[EPC];
+            Elem<T>::unpack(u, x);
+            int j = EPC - 1;
+#pragma unroll
+            for (int i = EPC - 2; i >= 0; --i) if (x[i] == m) j = i;
+            p.idx = (int)(lead + first_chunk * EPC + j);
+        }
+        if (split == 0) {            // unaligned head and tail, a handful of elements
+            for (int64_t e = tid; e < lead; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
+            for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
+        }
+    } else {
+        // Noise path: 4 more bytes per element and a true division; element-wise.
+        const int64_t ebeg = (split == 0) ? 0 : lead + cbeg * EPC;
+        const int64_t eend = (split == nsplit - 1) ? vocab : lead + cend * EPC;
+        for (int64_t e = ebeg + tid; e < eend; e += kThreads)
+            visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, np[e]);
+    }
+
+    // Wavefront reduction, then across the workgroup's wavefronts through LDS.
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const Partial o = shfl_xor(p, off, NOISE);
+        combine(p, o, c, NOISE);
+    }
+    __shared__ Partial wave_part[kThreads / mdx::kWave];
+    if ((tid & (mdx::kWave - 1)) == 0) wave_part[tid / mdx::kWave] = p;
+    __syncthreads();
+    if (tid == 0) {
+        Partial r = wave_part[0];
+#pragma unroll
+        for (int w = 1; w < kThreads / mdx::kWave; ++w) combine(r, wave_part[w], c, NOISE);
+        if (nsplit > 1) {
+            partials[row * nsplit + split] = r;
+        } else if (NOISE) {
+            x0[row] = r.pick_idx;
+            x0_p[row] = fast_exp2((r.pick_x - r.m) * c) / r.s;
+        } else {
+            x0[row] = r.idx;
+            x0_p[row] = 1.0f / r.s;
+        }
+    }
+}
+
+// Merges the row splits: one lane per row.
+template <bool NOISE>
+__global__ __launch_bounds__(kThreads) void confidence_finalize_kernel(
+    const Partial* __restrict__ partials, int nsplit,
+    const float* __restrict__ temperatures, int rows_per_temp,
+    int64_t rows, int64_t* __restrict__ x0, float* __restrict__ x0_p)
+{
+    const int64_t row = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (row >= rows) return;
+    const float T_ = temperatures ? temperatures[row / rows_per_temp] : 1.0f;
+    const float c = kLog2e / T_;
+    Partial r = partials[row * nsplit];
+    for (int s = 1; s < nsplit; ++s) combine(r, partials[row * nsplit + s], c, NOISE);
+    if (NOISE) {
+        x0[row] = r.pick_idx;
+        x0_p[row] = fast_exp2((r.pick_x - r.m) * c) / r.s;
+    } else {
+        x0[row] = r.idx;
+        x0_p[row] = 1.0f / r.s;
+    }
+}
+
+// One workgroup per sequence; lane p owns block position p.
+constexpr int kMaxBlockLen = 1024;
+__global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
+    const int64_t* __restrict__ x0, const float* __restrict__ x0_p, int64_t* __restrict__ tokens,
+    int64_t mask_token_id, float threshold, int k,
+    uint8_t* __restrict__ transfer, int32_t* __restrict__ count, int block_len)
+{
+    __shared__ float conf_s[kMaxBlockLen];
+    __shared__ int n_hi, n_masked, n_commit;
+    const int b = blockIdx.x;
+    const int p = threadIdx.x;
+    const bool on = p < block_len;
+    const int64_t at = (int64_t)b * block_len + p;
+    if (p == 0) { n_hi = 0; n_masked = 0; n_commit = 0; }
+    __syncthreads();
+    const bool masked = on && tokens[at] == mask_token_id;
+    const float conf = masked ? x0_p[at] : -INFINITY;
+    const bool hi = conf > threshold;
+    if (on) conf_s[p] = conf;
+    if (hi) atomicAdd(&n_hi, 1);
+    if (masked) atomicAdd(&n_masked, 1);
+    __syncthreads();
+    bool commit;
+    if (n_hi >= k) {
+        commit = hi;
+    } else {
+        // rank among masked positions: higher confidence first, lower position first on ties
+        int rank = 0;
+        if (masked) {
+            for (int j = 0; j < block_len; ++j) {
+                const float cj = conf_s[j];
+                rank += (cj > conf || (cj == conf && j < p)) ? 1 : 0;
+            }
+        }
+        commit = masked && rank < k;     // at most min(k, n_masked) positions
+    }
+    if (on) {
+        transfer[at] = commit ? 1 : 0;
+        if (commit) {
+            tokens[at] = x0[at];
+            atomicAdd(&n_commit, 1);
+        }
+    }
+    __syncthreads();
+    if (p == 0) count[b] = n_commit;
+}
+
+// Splits per row so that small batches still fill the chip: target >= ~2 waves of workgroups
+// while keeping at least 32 KiB of logits per workgroup.
+int pick_nsplit(int64_t rows, int64_t vocab) {
+    const int64_t target = 2048;
+    int64_t n = (target + rows - 1) / rows;
+    const int64_t max_by_size = vocab / 16384 > 0 ? vocab / 16384 : 1;
+    if (n > max_by_size) n = max_by_size;
+    if (n < 1) n = 1;
+    if (n > 64) n = 64;
+    return (int)n;
+}
+
+template <typename T>
+int launch_confidence(const void* logits, int64_t row_stride, const float* temperatures, int rows_per_temp,
+                      const float* noise, int64_t noise_row_stride, int64_t* x0, float* x0_p,
+                      int64_t rows, int64_t vocab, int nsplit, Partial* partials, hipStream_t stream)
+{
+    const dim3 grid((unsigned)rows, (unsigned)nsplit);
+    if (noise)
+        confidence_argmax_kernel<T, true><<<grid, kThreads, 0, stream>>>(
+            (const T*)logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, vocab, nsplit, partials, x0, x0_p);
+    else
+        confidence_argmax_kernel<T, false><<<grid, kThreads, 0, stream>>>(
+            (const T*)logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, vocab, nsplit, partials, x0, x0_p);
+    int rc = mdx::check_launch("confidence_argmax");
+    if (rc != MDX_OK || nsplit == 1) return rc;
+    const unsigned fgrid = (unsigned)((rows + kThreads - 1) / kThreads);
+    if (noise)
+        confidence_finalize_kernel<true><<<fgrid, kThreads, 0, stream>>>(partials, nsplit, temperatures, rows_per_temp, rows, x0, x0_p);
+    else
+        confidence_finalize_kernel<false><<<fgrid, kThreads, 0, stream>>>(partials, nsplit, temperatures, rows_per_temp, rows, x0, x0_p);
+    return mdx::check_launch("confidence_finalize");
+}
+
+}  // namespace
+
+extern "C" int64_t mdx_confidence_argmax_workspace_bytes(int64_t rows, int64_t vocab) {
+    if (rows <= 0 || vocab <= 0) return 0;
+    const int nsplit = pick_nsplit(rows, vocab);
+    return nsplit > 1 ? rows * nsplit * (int64_t)sizeof(Partial) : 0;
+}
+
+extern "C" int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
+                                     const float* temperatures, int32_t rows_per_temp,
+                                     const float* noise, int64_t noise_row_stride,
+                                     int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
+                                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MDX_REQUIRE(rows >= 0 && vocab >= 0, MDX_EINVAL, "confidence_argmax: negative size");
+    if (rows == 0) return MDX_OK;
+    MDX_REQUIRE(vocab > 0, MDX_EINVAL, "confidence_argmax: empty vocabulary");
+    MDX_REQUIRE(logits && x0 && x0_p, MDX_EINVAL, "confidence_argmax: null pointer");
+    MDX_REQUIRE(vocab < (int64_t)0x7fffffff && rows < (int64_t)0x7fffffff, MDX_EUNSUPPORTED,
+                "confidence_argmax: rows %lld or vocab %lld out of range", (long long)rows, (long long)vocab);
+    MDX_REQUIRE(row_stride >= vocab, MDX_EUNSUPPORTED, "confidence_argmax: row_stride %lld < vocab %lld", (long long)row_stride, (long long)vocab);
+    MDX_REQUIRE(!temperatures || rows_per_temp > 0, MDX_EINVAL, "confidence_argmax: rows_per_temp must be positive");
+    MDX_REQUIRE(!noise || noise_row_stride >= vocab, MDX_EINVAL, "confidence_argmax: noise_row_stride < vocab");
+    const int esz = dtype == MDX_F32 ? 4 : 2;
+    MDX_REQUIRE((reinterpret_cast<uintptr_t>(logits) % esz) == 0, MDX_EUNSUPPORTED, "confidence_argmax: logits not element-aligned");
+    const int nsplit = pick_nsplit(rows, vocab);
+    const int64_t need = nsplit > 1 ? rows * nsplit * (int64_t)sizeof(Partial) : 0;
+    MDX_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), MDX_EWORKSPACE,
+                "confidence_argmax: workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
+    Partial* partials = static_cast<Partial*>(workspace);
+    switch (dtype) {
+        case MDX_BF16: return launch_confidence<__bf16>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
+        case MDX_F16:  return launch_confidence<__half>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
+        case MDX_F32:  return launch_confidence<float>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
+        default: return mdx::fail(MDX_EUNSUPPORTED, "confidence_argmax: dtype %d", dtype);
+    }
+}
+
+extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t* tokens,
+                                   int64_t mask_token_id, float threshold, int32_t k,
+                                   uint8_t* transfer, int32_t* count,
+                                   int32_t bs, int32_t block_len, mdx_stream_t stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    MDX_REQUIRE(bs >= 0 && block_len >= 0, MDX_EINVAL, "select_transfer: negative size");
+    if (bs == 0 || block_len == 0) return MDX_OK;
+    MDX_REQUIRE(x0 && x0_p && tokens && transfer && count, MDX_EINVAL, "select_transfer: null pointer");
+    MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "select_transfer: block_len %d > %d", block_len, kMaxBlockLen);
+    MDX_REQUIRE(k >= 1, MDX_EINVAL, "select_transfer: k %d < 1", k);
+    const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
+    select_transfer_kernel<<<(unsigned)bs, threads, 0, stream>>>(x0, x0_p, tokens, mask_token_id, threshold, k, transfer, count, block_len);
+    return mdx::check_launch("select_transfer");
+}
+
+extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
+                               const float* temperatures, const float* noise, int64_t noise_row_stride,
+                               int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                               int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                               int32_t bs, int32_t block_len, int64_t vocab,
+                               void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    MDX_REQUIRE(bs >= 0 && block_len >= 0, MDX_EINVAL, "unmask_step: negative size");
+    MDX_REQUIRE(k >= 1, MDX_EINVAL, "unmask_step: k %d < 1", k);
+    MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "unmask_step: block_len %d > %d", block_len, kMaxBlockLen);
+    if (bs == 0 || block_len == 0) return MDX_OK;
+    MDX_REQUIRE(tokens && transfer && count, MDX_EINVAL, "unmask_step: null pointer");
+    int rc = mdx_confidence_argmax(logits, row_stride, dtype, temperatures, block_len, noise, noise_row_stride,
+                                   x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, stream);
+    if (rc != MDX_OK) return rc;
+    return mdx_select_transfer(x0, x0_p, tokens, mask_token_id, threshold, k, transfer, count, bs, block_len, stream);
+}

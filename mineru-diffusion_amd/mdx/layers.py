@@ -1,0 +1,73 @@
+"""The two layers that own the hot path, as the engine defines them."""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .context import get_context
+from .ops import flash_attn_with_kvcache, sparse_attn_varlen, store_kvcache_maybe4d, unmask_step
+
+
+class Attention(nn.Module):
+    """nanovllm/layers/sdar_attention.py:19-57: store the step's K/V into the paged cache,
+    then staircase attention over the packed prompt (prefill) or non-causal attention of
+    the current block over the cache (decode).  Inputs arrive through the global Context."""
+
+    def __init__(self, num_heads, head_dim, scale, num_kv_heads):
+        super().__init__()
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.scale = scale
+        self.num_kv_heads = num_kv_heads
+        self.k_cache = self.v_cache = torch.tensor([])
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+        context = get_context()
+        k_cache, v_cache = self.k_cache, self.v_cache
+        if k_cache.numel() and v_cache.numel():
+            store_kvcache_maybe4d(k, v, k_cache, v_cache, context.slot_mapping)
+        if context.is_prefill:
+            o = sparse_attn_varlen(q, k, v, cu_seqlens_q=context.cu_seqlens_q, cu_seqlens_k=context.cu_seqlens_k,
+                                   staircase_size=context.block_size,
+                                   max_seqlen=context.max_seqlen_k or None, softmax_scale=self.scale)
+            o = o.flatten(1)
+        else:
+            o = flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=context.context_lens,
+                                        block_table=context.block_tables, softmax_scale=self.scale, causal=False)
+            o = o.flatten(2)
+        return o
+
+
+class Sampler(nn.Module):
+    """nanovllm/layers/sampler.py:6-61.  The device does the whole step (confidence, argmax,
+    selection); only the [bs, S] results cross to the host to update the Sequence objects.
+
+    `k` is the number of positions committed when fewer than k exceed the threshold
+    (1 = the engine's rule, sampler.py:44-50).  `noise_fn(logits) -> fp32 noise` supplies the
+    Gumbel term of sampler.py:15-18 when sampling is wanted; None = plain argmax."""
+
+    def __init__(self, k: int = 1, noise_fn=None):
+        super().__init__()
+        self.k = k
+        self.noise_fn = noise_fn
+
+    def prepare(self, logits: torch.Tensor, temperatures: torch.Tensor):
+        from .ops import confidence_argmax
+        noise = self.noise_fn(logits) if self.noise_fn is not None else None
+        return confidence_argmax(logits, temperatures, noise)
+
+    def forward(self, logits: torch.Tensor, temperatures: torch.Tensor, seqs) -> int:
+        strategy = seqs[0].sampling_params.denoising_strategy
+        if strategy != 'low_confidence_dynamic':
+            raise NotImplementedError(f"Denoising strategy {strategy} not implemented")
+        threshold = seqs[0].sampling_params.dynamic_threshold
+        x = torch.stack([seq.current_denoising_block for seq in seqs], dim=0).to(logits.device)
+        noise = self.noise_fn(logits) if self.noise_fn is not None else None
+        _, _, transfer, count = unmask_step(logits, x, seqs[0].mask_token_id, threshold, self.k,
+                                            temperatures=temperatures, noise=noise)
+        x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
+        for i, seq in enumerate(seqs):
+            seq.current_denoising_block = x_cpu[i]
+            seq.current_step_map[transfer_cpu[i]] = seq.current_denoise_step
+            seq.current_denoise_step += 1
+        return int(count.sum().item())

@@ -1,0 +1,226 @@
+"""The reference's hot-path functions, same signatures, running in libmdx.so.
+
+Tensors must live on the GPU; every kernel is enqueued on torch's current
+stream, allocates nothing itself (outputs and workspaces come from torch's
+caching allocator, so the calls are safe under graph capture) and never
+synchronises.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from ._lib import MdxError, check
+
+_DTYPES = {torch.bfloat16: _lib.MDX_BF16, torch.float16: _lib.MDX_F16, torch.float32: _lib.MDX_F32}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise MdxError("mdx ops run on the GPU only: got a tensor on " + str(t.device))
+
+
+def _i32(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype != torch.int32:
+        raise MdxError(f"{what} must be int32, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+# --------------------------------------------------------------------------- store_kvcache
+def store_kvcache(key: torch.Tensor, value: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  slot_mapping: torch.Tensor) -> None:
+    """nanovllm/layers/attention.py:33-40: key/value [N, Hkv, d] (row stride free, rows dense),
+    caches [pages, page, Hkv, d], slot_mapping [N] int32 with -1 = skip.  In place."""
+    _need_gpu(key, value, k_cache, v_cache, slot_mapping)
+    N, num_heads, head_dim = key.shape
+    D = num_heads * head_dim
+    assert key.stride(-1) == 1 and value.stride(-1) == 1
+    assert key.stride(1) == head_dim and value.stride(1) == head_dim
+    assert k_cache.stride(1) == D and v_cache.stride(1) == D
+    assert slot_mapping.numel() == N
+    assert key.dtype == value.dtype == k_cache.dtype == v_cache.dtype
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    slots = _i32(slot_mapping, "slot_mapping")
+    num_slots = k_cache.numel() // D
+    rc = _lib.lib().mdx_store_kvcache(key.data_ptr(), value.data_ptr(), key.stride(0), value.stride(0),
+                                      k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(),
+                                      N, D, key.element_size(), num_slots, _stream(key))
+    check(rc, "store_kvcache")
+
+
+def store_kvcache_maybe4d(k, v, k_cache, v_cache, slot_mapping) -> None:
+    """nanovllm/layers/sdar_attention.py:11-16: [b, s, h, d] inputs are flattened to [(b s), h, d]."""
+    if k.dim() == 4:
+        k = k.reshape(-1, k.shape[2], k.shape[3]) if k.is_contiguous() else k.flatten(0, 1)
+        v = v.reshape(-1, v.shape[2], v.shape[3]) if v.is_contiguous() else v.flatten(0, 1)
+        slot_mapping = slot_mapping.reshape(-1)
+    store_kvcache(k, v, k_cache, v_cache, slot_mapping)
+
+
+# --------------------------------------------------------------------------- staircase prefill
+def sparse_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
+                       cu_seqlens_k: torch.Tensor, staircase_size: int = 4, *, max_seqlen: int | None = None,
+                       softmax_scale: float | None = None) -> torch.Tensor:
+    """block_prefill_attention_v2.py:168-202: q [N, Hq, d], k/v [N, Hkv, d] packed over
+    sequences, cu_seqlens int32 [B+1], blocks of `staircase_size` right-aligned; returns o like q.
+    max_seqlen (keyword, optional) only sizes the grid; the engine has it in its Context."""
+    _need_gpu(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    assert q.dim() == k.dim() == v.dim() == 3
+    assert q.shape[0] == k.shape[0] == v.shape[0]
+    assert k.shape[1] == v.shape[1] and k.shape[2] == v.shape[2]
+    assert q.shape[2] == k.shape[2]
+    assert q.shape[1] % k.shape[1] == 0
+    assert staircase_size in [1, 2, 4, 8, 16, 32, 64, 128]
+    assert q.dtype == k.dtype == v.dtype
+    total, hq, d = q.shape
+    hkv = k.shape[1]
+    # strided views (e.g. slices of a fused QKV projection) are read in place
+    q, k, v = (t if t.stride(-1) == 1 else t.contiguous() for t in (q, k, v))
+    o = torch.empty((total, hq, d), dtype=q.dtype, device=q.device)
+    cu_q, cu_k = _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(cu_seqlens_k, "cu_seqlens_k")
+    batch = cu_k.numel() - 1
+    scale = 1.0 / math.sqrt(d) if softmax_scale is None else float(softmax_scale)
+    rc = _lib.lib().mdx_staircase_attn_varlen(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+        q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), o.stride(0), o.stride(1),
+        cu_q.data_ptr(), cu_k.data_ptr(), batch, int(max_seqlen) if max_seqlen else total, total,
+        hq, hkv, d, staircase_size, scale, _DTYPES[q.dtype], _stream(q))
+    check(rc, "sparse_attn_varlen")
+    return o
+
+
+sparse_attn_varlen_v2 = sparse_attn_varlen
+
+
+# --------------------------------------------------------------------------- paged decode
+def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
+                            cache_seqlens: torch.Tensor, block_table: torch.Tensor,
+                            softmax_scale: float | None = None, causal: bool = False) -> torch.Tensor:
+    """The subset of flash_attn.flash_attn_with_kvcache used at sdar_attention.py:50-55:
+    q [bs, Sq, Hq, d], caches [pages, page, Hkv, d], block_table [bs, max_pages] int32,
+    cache_seqlens [bs] int32, non-causal.  Returns o like q."""
+    if causal:
+        raise MdxError("flash_attn_with_kvcache: only causal=False (block-diffusion decode) is implemented")
+    _need_gpu(q, k_cache, v_cache, cache_seqlens, block_table)
+    assert q.dim() == 4 and k_cache.dim() == 4 and v_cache.shape == k_cache.shape
+    assert q.dtype == k_cache.dtype == v_cache.dtype
+    bs, sq, hq, d = q.shape
+    num_pages, page, hkv, _ = k_cache.shape
+    if q.stride(-1) != 1:
+        q = q.contiguous()
+    assert k_cache.stride(-1) == 1 and v_cache.stride() == k_cache.stride()
+    bt, lens = _i32(block_table, "block_table"), _i32(cache_seqlens, "cache_seqlens")
+    assert bt.dim() == 2 and bt.shape[0] == bs and lens.numel() == bs
+    o = torch.empty((bs, sq, hq, d), dtype=q.dtype, device=q.device)
+    L = _lib.lib()
+    ws_bytes = L.mdx_paged_block_attn_workspace_bytes(bs, sq, hq, hkv, d, bt.shape[1], page)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+    scale = 1.0 / math.sqrt(d) if softmax_scale is None else float(softmax_scale)
+    rc = L.mdx_paged_block_attn(
+        q.data_ptr(), o.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+        q.stride(0), q.stride(1), q.stride(2), o.stride(0), o.stride(1), o.stride(2),
+        k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+        bt.data_ptr(), bt.stride(0), lens.data_ptr(),
+        bs, sq, hq, hkv, d, bt.shape[1], page, num_pages, scale, _DTYPES[q.dtype],
+        ws.data_ptr(), ws_bytes, _stream(q))
+    check(rc, "flash_attn_with_kvcache")
+    return o
+
+
+# --------------------------------------------------------------------------- unmask step
+def _logits2d(logits: torch.Tensor) -> torch.Tensor:
+    if logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    v = logits.shape[-1]
+    l2 = logits.reshape(-1, v) if logits.dim() != 2 else logits
+    return l2
+
+
+def confidence_argmax(logits: torch.Tensor, temperatures: torch.Tensor | None = None,
+                      noise: torch.Tensor | None = None):
+    """Sampler.prepare (nanovllm/layers/sampler.py:11-22) without its internal RNG:
+    logits [bs, S, V], temperatures [bs] or [bs, 1] fp32 -> (x0 int64 [bs, S], x0_p fp32 [bs, S]).
+    `noise` ([bs, S, V] fp32) is added to logits/T before the argmax; None = plain argmax."""
+    _need_gpu(logits, temperatures, noise)
+    lead = logits.shape[:-1]
+    l2 = _logits2d(logits)
+    rows, vocab = l2.shape
+    rows_per_temp = 1
+    t_ptr = None
+    if temperatures is not None:
+        temperatures = temperatures.reshape(-1).to(torch.float32).contiguous()
+        assert rows % temperatures.numel() == 0
+        rows_per_temp = rows // temperatures.numel()
+        t_ptr = temperatures.data_ptr()
+    n_ptr, n_stride = None, 0
+    if noise is not None:
+        noise = noise.reshape(rows, vocab).to(torch.float32).contiguous()
+        n_ptr, n_stride = noise.data_ptr(), noise.stride(0)
+    x0 = torch.empty(rows, dtype=torch.int64, device=logits.device)
+    x0_p = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    L = _lib.lib()
+    ws_bytes = L.mdx_confidence_argmax_workspace_bytes(rows, vocab)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=logits.device)
+    rc = L.mdx_confidence_argmax(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, rows_per_temp, n_ptr, n_stride,
+                                 x0.data_ptr(), x0_p.data_ptr(), rows, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    check(rc, "confidence_argmax")
+    return x0.view(lead), x0_p.view(lead)
+
+
+def select_transfer(x0: torch.Tensor, x0_p: torch.Tensor, tokens: torch.Tensor, mask_token_id: int,
+                    threshold: float, k: int = 1):
+    """Device form of the selection loop (sampler.py:32-54, modeling_mineru_diffusion.py:518-532).
+    tokens [bs, S] int64 is updated in place; returns (transfer bool [bs, S], count int32 [bs])."""
+    _need_gpu(x0, x0_p, tokens)
+    assert tokens.dtype == torch.int64 and x0.dtype == torch.int64 and x0_p.dtype == torch.float32
+    assert tokens.is_contiguous() and x0.is_contiguous() and x0_p.is_contiguous()
+    bs, S = tokens.shape
+    transfer = torch.empty((bs, S), dtype=torch.uint8, device=tokens.device)
+    count = torch.empty(bs, dtype=torch.int32, device=tokens.device)
+    rc = _lib.lib().mdx_select_transfer(x0.data_ptr(), x0_p.data_ptr(), tokens.data_ptr(), int(mask_token_id),
+                                        float(threshold), int(k), transfer.data_ptr(), count.data_ptr(), bs, S,
+                                        _stream(tokens))
+    check(rc, "select_transfer")
+    return transfer.view(torch.bool), count
+
+
+def unmask_step(logits: torch.Tensor, tokens: torch.Tensor, mask_token_id: int, threshold: float, k: int = 1,
+                temperatures: torch.Tensor | None = None, noise: torch.Tensor | None = None):
+    """One whole unmask step on the device: logits [bs, S, V], tokens [bs, S] int64 (in place).
+    Returns (x0, x0_p, transfer, count)."""
+    _need_gpu(logits, tokens, temperatures, noise)
+    assert tokens.dtype == torch.int64 and tokens.is_contiguous()
+    bs, S = tokens.shape
+    l2 = _logits2d(logits)
+    rows, vocab = l2.shape
+    assert rows == bs * S
+    t_ptr = None
+    if temperatures is not None:
+        temperatures = temperatures.reshape(-1).to(torch.float32).contiguous()
+        assert temperatures.numel() == bs
+        t_ptr = temperatures.data_ptr()
+    n_ptr, n_stride = None, 0
+    if noise is not None:
+        noise = noise.reshape(rows, vocab).to(torch.float32).contiguous()
+        n_ptr, n_stride = noise.data_ptr(), noise.stride(0)
+    dev = logits.device
+    x0 = torch.empty((bs, S), dtype=torch.int64, device=dev)
+    x0_p = torch.empty((bs, S), dtype=torch.float32, device=dev)
+    transfer = torch.empty((bs, S), dtype=torch.uint8, device=dev)
+    count = torch.empty(bs, dtype=torch.int32, device=dev)
+    L = _lib.lib()
+    ws_bytes = L.mdx_confidence_argmax_workspace_bytes(rows, vocab)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    rc = L.mdx_unmask_step(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, n_ptr, n_stride,
+                           tokens.data_ptr(), int(mask_token_id), float(threshold), int(k),
+                           x0.data_ptr(), x0_p.data_ptr(), transfer.data_ptr(), count.data_ptr(),
+                           bs, S, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    check(rc, "unmask_step")
+    return x0, x0_p, transfer.view(torch.bool), count

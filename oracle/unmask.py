@@ -1,0 +1,85 @@
+"""Oracle: the per-block confidence unmask step.  Test infrastructure only.
+
+Reference followed:
+  engines/nano_dvlm/nanovllm/layers/sampler.py:11-61            (engine variant)
+  mineru_diffusion/modeling_mineru_diffusion.py:518-532,602-623,702-719 (HF variant)
+"""
+from __future__ import annotations
+
+import numpy as np
+
+
+def num_transfer_tokens(block_length: int, steps: int) -> list[int]:
+    """modeling_mineru_diffusion.py:617-623: block_length split over steps, the
+    remainder given to the first steps."""
+    base, rem = divmod(block_length, steps)
+    return [base + (1 if i < rem else 0) for i in range(steps)]
+
+
+def confidence_argmax(logits: np.ndarray, temperatures=None, noise: np.ndarray | None = None):
+    """logits [bs, S, V] (any float dtype, already widened to >= fp32 by the caller),
+    temperatures [bs] or None (= 1) -> (x0 int64 [bs, S], x0_p float64 [bs, S]).
+
+    sampler.py:13  l = logits.float() / T          (fp32 division)
+    sampler.py:15-18  x0 = argmax(l + noise); noise is an explicit input here,
+                      None = plain argmax (first index on ties, as torch.argmax)
+    sampler.py:20-21  x0_p = softmax(l)[x0]        (summed in fp64 here)
+    """
+    l32 = np.asarray(logits, dtype=np.float32)
+    if temperatures is not None:
+        t = np.asarray(temperatures, dtype=np.float32).reshape(-1, 1, 1)
+        l32 = (l32 / t).astype(np.float32)
+    pick = l32 if noise is None else (l32 + np.asarray(noise, dtype=np.float32)).astype(np.float32)
+    x0 = pick.argmax(axis=-1).astype(np.int64)          # numpy: first occurrence
+    l64 = l32.astype(np.float64)
+    m = l64.max(axis=-1, keepdims=True)
+    e = np.exp(l64 - m)
+    chosen = np.take_along_axis(e, x0[..., None], axis=-1)[..., 0]
+    return x0, chosen / e.sum(axis=-1)
+
+
+def select_transfer(conf: np.ndarray, masked: np.ndarray, threshold: float, k: int) -> np.ndarray:
+    """conf [bs, S] float, masked [bs, S] bool -> transfer [bs, S] bool.
+
+    confidence = where(masked, conf, -inf)            (modeling:708, sampler.py:39)
+    hi = confidence > threshold (strict)              (modeling:526, sampler.py:44)
+    if hi.sum() >= k: commit all of hi                (modeling:527-529)
+    else: commit the k most confident masked positions (modeling:530-531)
+
+    Defined here where the reference leaves it open: among equal confidences the
+    LOWER position wins, and at most #masked positions are committed (the
+    reference's topk would otherwise return already-committed -inf positions).
+    The engine variant (sampler.py:41-50: skip rows without masked positions,
+    all of hi if any else top-1) is this rule with k = 1.
+    """
+    conf = np.asarray(conf)
+    masked = np.asarray(masked, dtype=bool)
+    out = np.zeros(conf.shape, dtype=bool)
+    for b in range(conf.shape[0]):
+        c = np.where(masked[b], conf[b].astype(np.float64), -np.inf)
+        hi = c > threshold
+        if hi.sum() >= k:
+            out[b] = hi
+            continue
+        want = min(k, int(masked[b].sum()))
+        taken = np.zeros_like(hi)
+        for _ in range(want):
+            best = -1
+            for p in range(c.shape[0]):
+                if masked[b, p] and not taken[p] and (best < 0 or c[p] > c[best]):
+                    best = p
+            taken[best] = True
+        out[b] = taken
+    return out
+
+
+def unmask_step(logits: np.ndarray, tokens: np.ndarray, mask_token_id: int, threshold: float, k: int,
+                temperatures=None, noise=None):
+    """One unmask step on identical logits: returns (x0, x0_p, transfer, new_tokens).
+    masked = tokens == mask_token_id (sampler.py:32); x[transfer] = x0[transfer]
+    (sampler.py:54, modeling:717)."""
+    x0, x0_p = confidence_argmax(logits, temperatures, noise)
+    masked = np.asarray(tokens) == mask_token_id
+    transfer = select_transfer(x0_p.astype(np.float32), masked, threshold, k)
+    new_tokens = np.where(transfer, x0, np.asarray(tokens)).astype(np.int64)
+    return x0, x0_p, transfer, new_tokens

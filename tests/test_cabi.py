@@ -1,0 +1,95 @@
+"""The C ABI without a GPU: the library loads, exports every symbol include/mdx.h declares,
+and refuses bad arguments before launching anything."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def L():
+    import mdx
+    if not mdx.library_path().exists():
+        from importlib import import_module
+        import sys
+        sys.path.insert(0, str(ROOT))
+        import_module("__graft_entry__").build()
+    return mdx.lib()
+
+
+def _declared():
+    text = (ROOT / "include" / "mdx.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mdx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree(L):
+    from mdx import _lib
+    names = _declared()
+    assert names, "no declarations found in include/mdx.h"
+    assert sorted(_lib.SIGNATURES) == names
+    for n in names:
+        assert hasattr(L, n), f"libmdx.so does not export {n}"
+
+
+def test_version_matches_header(L):
+    text = (ROOT / "include" / "mdx.h").read_text()
+    assert L.mdx_version() == int(re.search(r"#define MDX_VERSION (\d+)", text).group(1))
+
+
+def test_workspace_queries_are_pure_host_arithmetic(L):
+    assert L.mdx_confidence_argmax_workspace_bytes(1024, 151936) == 0 or \
+        L.mdx_confidence_argmax_workspace_bytes(1024, 151936) % 24 == 0
+    few = L.mdx_confidence_argmax_workspace_bytes(32, 151936)
+    assert few > 0 and few % (32 * 24) == 0            # small batches split rows over workgroups
+    ws = L.mdx_paged_block_attn_workspace_bytes(16, 32, 16, 8, 128, 17, 256)
+    assert ws > 0 and ws % (16 * 16 * 32 * 130 * 4) == 0
+    assert L.mdx_paged_block_attn_workspace_bytes(0, 32, 16, 8, 128, 17, 256) == 0
+
+
+def test_bad_arguments_are_refused_without_a_launch(L):
+    null = None
+    one = ctypes.c_void_p(16)     # never dereferenced: every call below must fail validation first
+    assert L.mdx_store_kvcache(null, null, 0, 0, null, null, null, 5, 1024, 2, 10, null) == -1
+    assert b"null" in L.mdx_last_error()
+    assert L.mdx_store_kvcache(one, one, 0, 0, one, one, one, 5, 1024, 3, 10, null) == -2
+    assert L.mdx_store_kvcache(null, null, 0, 0, null, null, null, 0, 1024, 2, 10, null) == 0   # empty: no-op
+    sa = lambda **kw: L.mdx_staircase_attn_varlen(                                            # noqa: E731
+        one, one, one, one, 2048, 128, 1024, 128, 1024, 128, 2048, 128, one, one, 1, 100, 100,
+        kw.get("hq", 16), kw.get("hkv", 8), kw.get("d", 128), kw.get("S", 32), kw.get("scale", 0.1), kw.get("dtype", 0), null)
+    assert sa(d=64) == -2 and b"head_dim" in L.mdx_last_error()
+    assert sa(S=48) == -1 and b"staircase_size" in L.mdx_last_error()
+    assert sa(hq=12) == -1
+    assert sa(dtype=1) == -2
+    assert sa(scale=-1.0) == -1
+    pa = lambda **kw: L.mdx_paged_block_attn(                                                  # noqa: E731
+        one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,
+        4, kw.get("sq", 32), 16, 8, 128, 17, kw.get("page", 256), 100, 0.1, 0, kw.get("ws", null), kw.get("ws_bytes", 0), null)
+    assert pa(sq=33) == -2
+    assert pa(page=100) == -2
+    assert pa() == -3 and b"workspace" in L.mdx_last_error()
+    assert L.mdx_select_transfer(one, one, one, 7, 0.9, 0, one, one, 2, 32, null) == -1       # k < 1
+    assert L.mdx_select_transfer(one, one, one, 7, 0.9, 1, one, one, 2, 2000, null) == -2      # block too long
+    assert L.mdx_confidence_argmax(one, 10, 0, null, 1, null, 0, one, one, 4, 20, null, 0, null) == -2   # stride < vocab
+
+
+def test_ops_fail_loudly_off_gpu():
+    import torch
+    import mdx
+    x = torch.zeros(4, 8, 128, dtype=torch.bfloat16)
+    with pytest.raises(mdx.MdxError):
+        mdx.store_kvcache(x, x, torch.zeros(1, 256, 8, 128, dtype=torch.bfloat16),
+                          torch.zeros(1, 256, 8, 128, dtype=torch.bfloat16), torch.zeros(4, dtype=torch.int32))
+    with pytest.raises(mdx.MdxError):
+        mdx.sparse_attn_varlen(x, x, x, torch.tensor([0, 4], dtype=torch.int32), torch.tensor([0, 4], dtype=torch.int32), 32)
+
+
+def test_context_mirror():
+    import mdx
+    mdx.set_context(True, max_seqlen_q=5, block_size=32)
+    assert mdx.get_context().is_prefill and mdx.get_context().max_seqlen_q == 5
+    mdx.reset_context()
+    assert not mdx.get_context().is_prefill and mdx.get_context().slot_mapping is None

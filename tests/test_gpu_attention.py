@@ -1,0 +1,196 @@
+"""GPU parity: staircase block-prefill attention and paged single-block attention through
+the C ABI vs the fp32 oracle (torch SDPA with an explicit boolean mask).
+Tolerance: max-abs 2e-2 on bf16 outputs, the bound the task states for this path."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def _packed(g, lens, hq, hkv, d=128):
+    N = sum(lens)
+    q = torch.randn(N, hq, d, generator=g).bfloat16()
+    k = torch.randn(N, hkv, d, generator=g).bfloat16()
+    v = torch.randn(N, hkv, d, generator=g).bfloat16()
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    return q, k, v, cu
+
+
+def _check_prefill(dev, lens, S, hq=16, hkv=8, seed=0, max_seqlen=None):
+    import mdx
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, cu = _packed(g, lens, hq, hkv)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S, max_seqlen=max_seqlen)
+    torch.cuda.synchronize()
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
+    err = (o.float().cpu() - ref).abs().max().item()
+    assert err < TOL, f"max-abs {err} for lens={lens} S={S}"
+    return err
+
+
+@pytest.mark.parametrize("L", [1, 31, 32, 33, 64, 100, 127, 128, 129, 257, 1000])
+def test_prefill_single_sequence_block32(dev, L):
+    _check_prefill(dev, [L], 32, seed=L)
+
+
+@pytest.mark.parametrize("S", [1, 2, 4, 8, 16, 32, 64, 128])
+def test_prefill_all_staircase_sizes(dev, S):
+    _check_prefill(dev, [203, 77, 1, 160], S, seed=S)
+
+
+@pytest.mark.parametrize("hq,hkv", [(16, 8), (8, 8), (4, 1), (3, 1), (2, 2)])
+def test_prefill_gqa_ratios(dev, hq, hkv):
+    _check_prefill(dev, [150, 97], 32, hq=hq, hkv=hkv, seed=hq * 10 + hkv)
+
+
+def test_prefill_varlen_batch_with_empty_sequence(dev):
+    _check_prefill(dev, [300, 0, 45, 513, 32], 32, seed=42, max_seqlen=513)
+
+
+def test_prefill_reads_fused_qkv_views_in_place(dev):
+    """q, k, v as strided slices of one [N, (Hq+2Hkv)*d] projection output (sdar.py:73-78)."""
+    import mdx
+    g = torch.Generator().manual_seed(77)
+    N, hq, hkv, d = 333, 16, 8, 128
+    fused = torch.randn(N, (hq + 2 * hkv) * d, generator=g).bfloat16()
+    q = fused[:, :hq * d].view(N, hq, d)
+    k = fused[:, hq * d:(hq + hkv) * d].view(N, hkv, d)
+    v = fused[:, (hq + hkv) * d:].view(N, hkv, d)
+    cu = torch.tensor([0, 200, N], dtype=torch.int32)
+    dfused = fused.to(dev)
+    dq = dfused[:, :hq * d].view(N, hq, d)
+    dk = dfused[:, hq * d:(hq + hkv) * d].view(N, hkv, d)
+    dv = dfused[:, (hq + hkv) * d:].view(N, hkv, d)
+    o = mdx.sparse_attn_varlen(dq, dk, dv, cu.to(dev), cu.to(dev), 32)
+    torch.cuda.synchronize()
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
+
+
+def test_prefill_long_sequences(dev):
+    """Config-3-like lengths (non-multiples of 32 included), checked on whole outputs."""
+    err = _check_prefill(dev, [2048 + 5, 1024, 3000], 32, seed=3, max_seqlen=3000)
+    assert err < TOL
+
+
+def test_prefill_block_independence_full_size(dev):
+    """Size-independent property at full length: the outputs of the first blocks do not change
+    when later tokens change (block b never sees blocks > b)."""
+    import mdx
+    g = torch.Generator().manual_seed(5)
+    L, cut = 8192, 4096
+    q, k, v, cu = _packed(g, [L], 16, 8)
+    o1 = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    k2, v2, q2 = k.clone(), v.clone(), q.clone()
+    k2[cut:] = torch.randn(L - cut, 8, 128, generator=g).bfloat16()
+    v2[cut:] = torch.randn(L - cut, 8, 128, generator=g).bfloat16()
+    q2[cut:] = torch.randn(L - cut, 16, 128, generator=g).bfloat16()
+    o2 = mdx.sparse_attn_varlen(q2.to(dev), k2.to(dev), v2.to(dev), cu.to(dev), cu.to(dev), 32)
+    torch.cuda.synchronize()
+    assert torch.equal(o1[:cut], o2[:cut])
+    assert not torch.equal(o1[cut:], o2[cut:])
+    # and the last block against the oracle (it sees every key)
+    ref = oracle.masked_attention_f32(q[-32:], k, v, None, 1 / math.sqrt(128))
+    assert (o1[-32:].float().cpu() - ref).abs().max().item() < TOL
+
+
+def _paged_inputs(g, ctxs, sq=32, hq=16, hkv=8, d=128, page=256, pool=64):
+    bs = len(ctxs)
+    maxp = max(1, max((c + page - 1) // page for c in ctxs))
+    q = torch.randn(bs, sq, hq, d, generator=g).bfloat16()
+    kc = torch.randn(pool, page, hkv, d, generator=g).bfloat16()
+    vc = torch.randn(pool, page, hkv, d, generator=g).bfloat16()
+    perm = torch.randperm(pool, generator=g)
+    bt = torch.full((bs, maxp), -1, dtype=torch.int32)
+    at = 0
+    for b, c in enumerate(ctxs):
+        n = (c + page - 1) // page
+        bt[b, :n] = perm[at:at + n].to(torch.int32)
+        at += n
+    return q, kc, vc, bt, torch.tensor(ctxs, dtype=torch.int32)
+
+
+def _check_paged(dev, ctxs, seed=0, **kw):
+    import mdx
+    g = torch.Generator().manual_seed(seed)
+    q, kc, vc, bt, lens = _paged_inputs(g, ctxs, **kw)
+    scale = 1 / math.sqrt(q.shape[-1])
+    o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens.to(dev),
+                                    block_table=bt.to(dev), softmax_scale=scale, causal=False)
+    torch.cuda.synchronize()
+    ref = oracle.paged_block_attn(q, kc, vc, bt, lens, scale)
+    err = (o.float().cpu() - ref).abs().max().item()
+    assert err < TOL, f"max-abs {err} for ctxs={ctxs}"
+    return o
+
+
+@pytest.mark.parametrize("ctx", [1, 31, 32, 33, 127, 128, 129, 255, 256, 257, 544, 1000, 4128])
+def test_paged_single_sequence(dev, ctx):
+    _check_paged(dev, [ctx], seed=ctx)
+
+
+def test_paged_batch_with_padding_rows(dev):
+    o = _check_paged(dev, [544, 0, 4128, 1, 2000, 0, 777], seed=1)
+    assert o[1].abs().sum().item() == 0 and o[5].abs().sum().item() == 0
+
+
+@pytest.mark.parametrize("hq,hkv,sq", [(16, 8, 32), (8, 8, 32), (4, 1, 32), (16, 8, 7), (3, 1, 32)])
+def test_paged_head_layouts_and_short_blocks(dev, hq, hkv, sq):
+    _check_paged(dev, [300, 1500], seed=hq + sq, hq=hq, hkv=hkv, sq=sq)
+
+
+def test_paged_page_sizes(dev):
+    _check_paged(dev, [900, 130], seed=9, page=128, pool=32)
+    _check_paged(dev, [900, 130], seed=10, page=512, pool=8)
+
+
+def test_paged_is_invariant_to_page_placement(dev):
+    """Moving a sequence's pages elsewhere in the pool (and permuting its table) changes nothing."""
+    import mdx
+    g = torch.Generator().manual_seed(12)
+    q, kc, vc, bt, lens = _paged_inputs(g, [1500, 700], pool=32)
+    perm = torch.randperm(32, generator=g)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(32)
+    kc2, vc2 = kc[perm], vc[perm]                      # new pool: page j holds old page perm[j]
+    bt2 = torch.where(bt >= 0, inv[bt.clamp(min=0).long()].to(torch.int32), bt)
+    args = dict(cache_seqlens=lens.to(dev), softmax_scale=0.1, causal=False)
+    o1 = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), block_table=bt.to(dev), **args)
+    o2 = mdx.flash_attn_with_kvcache(q.to(dev), kc2.to(dev), vc2.to(dev), block_table=bt2.to(dev), **args)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
+
+
+def test_paged_config2_shape(dev):
+    """BASELINE config 2 shape: 16 sequences, prefix U[512, 4096] + 32, page 256 (small pool here)."""
+    g = torch.Generator().manual_seed(2)
+    ctxs = [int(x) + 32 for x in torch.randint(512, 4097, (16,), generator=g)]
+    _check_paged(dev, ctxs, seed=2, pool=300)
+
+
+def test_decode_matches_prefill_last_block(dev):
+    """Cross-check of the two kernels: prefill of (prefix + block) then decode of the same block over
+    the stored cache must agree (the decode block sees prefix + itself, as the last prefill block does)."""
+    import mdx
+    g = torch.Generator().manual_seed(31)
+    L, hq, hkv, d, page = 1000 + 32, 16, 8, 128, 256
+    q, k, v, cu = _packed(g, [L], hq, hkv)
+    dq, dk, dv, dcu = q.to(dev), k.to(dev), v.to(dev), cu.to(dev)
+    o_pre = mdx.sparse_attn_varlen(dq, dk, dv, dcu, dcu, 32)
+    pages = 8
+    kc = torch.zeros(pages, page, hkv, d, dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros_like(kc)
+    table = torch.tensor([[5, 2, 7, 0, 3]], dtype=torch.int32)
+    slots = torch.tensor(oracle.get_slots(table[0].tolist(), 0, L), dtype=torch.int32, device=dev)
+    mdx.store_kvcache(dk, dv, kc, vc, slots)
+    o_dec = mdx.flash_attn_with_kvcache(dq[-32:].unsqueeze(0), kc, vc,
+                                        cache_seqlens=torch.tensor([L], dtype=torch.int32, device=dev),
+                                        block_table=table.to(dev), softmax_scale=1 / math.sqrt(d), causal=False)
+    torch.cuda.synchronize()
+    assert (o_dec[0].float() - o_pre[-32:].float()).abs().max().item() < 1e-2

@@ -1,0 +1,141 @@
+"""Pins the KV-store, unmask and slot oracles against library routines and brute force."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+
+def test_store_matches_index_copy_and_leaves_the_rest():
+    g = torch.Generator().manual_seed(0)
+    N, hkv, d, pages, page = 50, 2, 8, 4, 32
+    key = torch.randn(N, hkv, d, generator=g)
+    val = torch.randn(N, hkv, d, generator=g)
+    kc0, vc0 = torch.randn(pages, page, hkv, d, generator=g), torch.randn(pages, page, hkv, d, generator=g)
+    slots = torch.randperm(pages * page, generator=g)[:N].to(torch.int32)
+    slots[::7] = -1
+    kc, vc = kc0.clone().numpy(), vc0.clone().numpy()
+    oracle.store_kvcache(key.numpy(), val.numpy(), kc, vc, slots.numpy())
+    keep = slots >= 0
+    want_k = kc0.clone().view(-1, hkv * d).index_copy_(0, slots[keep].long(), key.view(N, -1)[keep])
+    want_v = vc0.clone().view(-1, hkv * d).index_copy_(0, slots[keep].long(), val.view(N, -1)[keep])
+    assert np.array_equal(kc.reshape(-1, hkv * d), want_k.numpy())
+    assert np.array_equal(vc.reshape(-1, hkv * d), want_v.numpy())
+    untouched = np.setdiff1d(np.arange(pages * page), slots[keep].numpy())
+    assert np.array_equal(kc.reshape(-1, hkv * d)[untouched], kc0.view(-1, hkv * d).numpy()[untouched])
+
+
+def test_store_then_gather_round_trips_through_the_page_table():
+    g = torch.Generator().manual_seed(1)
+    L, hkv, d, page = 70, 2, 4, 16
+    table = [9, 3, 0, 5, 7]
+    k = torch.randn(L, hkv, d, generator=g)
+    kc, vc = np.zeros((12, page, hkv, d), np.float32), np.zeros((12, page, hkv, d), np.float32)
+    oracle.store_kvcache(k.numpy(), k.numpy(), kc, vc, np.array(oracle.get_slots(table, 0, L, page)))
+    assert torch.equal(oracle.paged_gather(torch.from_numpy(kc), table, L), k)
+
+
+def test_slots_brute_force_and_warmup():
+    table = [4, 1, 6]
+    for lo, hi in [(0, 0), (0, 5), (250, 262), (0, 768), (255, 257), (256, 512), (300, 301)]:
+        got = oracle.get_slots(table, lo, hi)
+        want = [table[t // 256] * 256 + t % 256 for t in range(lo, hi)]
+        assert got == want
+    assert oracle.get_slots([], 3, 8) == [-1] * 5
+
+
+def test_confidence_matches_torch_softmax_and_argmax():
+    g = torch.Generator().manual_seed(2)
+    logits = (torch.randn(3, 5, 777, generator=g) * 3).bfloat16()
+    temps = torch.tensor([0.5, 1.0, 3.0])
+    x0, p = oracle.confidence_argmax(logits.float().numpy(), temps.numpy())
+    l = logits.float() / temps.view(-1, 1, 1)
+    assert np.array_equal(x0, l.argmax(-1).numpy())
+    want = torch.softmax(l.double(), -1).gather(-1, l.argmax(-1, keepdim=True)).squeeze(-1)
+    np.testing.assert_allclose(p, want.numpy(), rtol=1e-12)
+    # conf of the argmax without noise is 1 / sum exp(l - max)
+    np.testing.assert_allclose(p, 1 / torch.exp(l.double() - l.double().amax(-1, keepdim=True)).sum(-1).numpy(), rtol=1e-12)
+
+
+def test_confidence_ties_take_the_first_index_and_noise_moves_the_pick():
+    logits = np.zeros((1, 2, 10), np.float32)
+    logits[0, 0, [3, 7]] = 5.0
+    x0, p = oracle.confidence_argmax(logits)
+    assert x0.tolist() == [[3, 0]]
+    assert torch.argmax(torch.from_numpy(logits), -1).tolist() == [[3, 0]]
+    noise = np.zeros_like(logits)
+    noise[0, 0, 8] = 100.0
+    x0n, pn = oracle.confidence_argmax(logits, None, noise)
+    assert x0n[0, 0] == 8
+    want = np.exp(0.0 - 5.0) / (2 + 8 * np.exp(-5.0))          # softmax WITHOUT the noise, at the noisy pick
+    np.testing.assert_allclose(pn[0, 0], want, rtol=1e-12)
+
+
+def test_num_transfer_tokens():
+    assert oracle.num_transfer_tokens(32, 8) == [4] * 8
+    assert oracle.num_transfer_tokens(32, 32) == [1] * 32
+    assert oracle.num_transfer_tokens(10, 4) == [3, 3, 2, 2]
+
+
+def _select_by_library(conf, masked, thr, k):
+    """The reference rule spelled with torch.topk (valid when there are no ties and >= k masked)."""
+    c = torch.where(torch.from_numpy(masked), torch.from_numpy(conf), torch.tensor(-torch.inf))
+    out = torch.zeros_like(c, dtype=torch.bool)
+    for b in range(c.shape[0]):
+        hi = c[b] > thr
+        if hi.sum() >= k:
+            out[b] = hi
+        else:
+            out[b, torch.topk(c[b], k).indices] = True
+    return out.numpy()
+
+
+@pytest.mark.parametrize("k", [1, 2, 4])
+def test_select_matches_topk_rule_on_tie_free_inputs(k):
+    rng = np.random.default_rng(k)
+    for trial in range(50):
+        conf = rng.random((4, 32)).astype(np.float32)          # distinct with probability 1
+        conf[0] *= 0.5                                         # row 0: nothing above 0.9
+        conf[1, :6] = 0.95 + 0.001 * np.arange(6)              # row 1: 6 above
+        masked = rng.random((4, 32)) < 0.7
+        masked[:, :8] = True                                   # at least 8 masked: topk never reaches -inf
+        got = oracle.select_transfer(conf, masked, 0.9, k)
+        assert np.array_equal(got, _select_by_library(conf, masked, 0.9, k))
+        assert not (got & ~masked).any()
+
+
+def test_select_brute_force_over_all_masks_on_six_positions():
+    conf = np.array([[0.95, 0.2, 0.91, 0.5, 0.7, 0.1]], np.float32)
+    for bits in itertools.product([False, True], repeat=6):
+        masked = np.array([bits])
+        for k in (1, 2, 3):
+            got = oracle.select_transfer(conf, masked, 0.9, k)[0]
+            idx = [i for i in range(6) if bits[i]]
+            hi = [i for i in idx if conf[0, i] > 0.9]
+            want = set(hi) if len(hi) >= k else set(sorted(idx, key=lambda i: -conf[0, i])[:k])
+            assert set(np.flatnonzero(got)) == want
+
+
+def test_select_strict_threshold_ties_and_engine_rule():
+    conf = np.array([[0.9, 0.9, 0.3, 0.3]], np.float32)
+    masked = np.ones((1, 4), bool)
+    # strict '>' : 0.9 is not above the 0.9 threshold -> top-k; equal values: lower position first
+    assert oracle.select_transfer(conf, masked, np.float32(0.9), 1).tolist() == [[True, False, False, False]]
+    assert oracle.select_transfer(conf, masked, np.float32(0.9), 3).tolist() == [[True, True, True, False]]
+    # engine rule = k 1: any above threshold -> all of them
+    assert oracle.select_transfer(conf, masked, 0.5, 1).tolist() == [[True, True, False, False]]
+    # rows without masked positions commit nothing (sampler.py:42-43)
+    assert not oracle.select_transfer(conf, np.zeros((1, 4), bool), 0.5, 1).any()
+
+
+def test_unmask_step_end_to_end_small():
+    g = torch.Generator().manual_seed(5)
+    logits = (torch.randn(2, 8, 50, generator=g) * 3).numpy()
+    tokens = np.full((2, 8), 99, np.int64)
+    tokens[0, :3] = [1, 2, 3]
+    x0, p, tr, new = oracle.unmask_step(logits, tokens, 99, 0.9, 2)
+    assert (new[0, :3] == [1, 2, 3]).all() and not tr[0, :3].any()
+    assert (new[tr] == x0[tr]).all() and (new[~tr] == tokens[~tr]).all()
+    assert tr.sum(-1).tolist() == [2, 2] or (p > 0.9).any()
