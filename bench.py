@@ -1,0 +1,344 @@
+"""Benchmark of the block-diffusion attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one prefill pass of the attention layer over BASELINE config 3 (8 packed
+sequences, lengths U[1024, 8192], 32-token blocks, Hq 16 / Hkv 8 / d 128, bf16):
+store_kvcache of the committed rows, then the staircase attention.  `value` is the
+attention's ALGORITHMIC throughput (4*d*Hq flops per visible (query, key) pair, masked
+pairs earn nothing) over the whole step time.  The same run also times, each with its own
+roofline entry under "ops": store_kvcache alone (config 3), the paged single-block attention
+(config 2) and the unmask step (config 4).  A bounded CPU leg runs the oracle (torch SDPA with
+an explicit boolean mask, index_copy-style store, fp64 softmax) on the host cores as a baseline.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+for p in (ROOT, ROOT / "mineru-diffusion_amd"):
+    if str(p) not in sys.path:
+        sys.path.insert(0, str(p))
+
+import numpy as np  # noqa: E402
+import torch  # noqa: E402
+
+HQ, HKV, D, S, PAGE, VOCAB, MASK_ID = 16, 8, 128, 32, 256, 151936, 151669
+PEAK_MFMA_TFLOPS = 2500.0          # MI355X dense bf16
+PEAK_HBM_GBS = 8000.0              # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def ev_pair():
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def time_kernel(fn, warmup, iters):
+    """Average duration (ms) of fn's GPU work, HIP events on the launch stream (torch's current
+    stream, which is where libmdx enqueues), one event pair per call."""
+    for _ in range(warmup):
+        fn(0)
+    torch.cuda.synchronize()
+    pairs = []
+    for i in range(iters):
+        a, b = ev_pair()
+        a.record()
+        fn(i)
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in pairs]
+    return float(np.mean(ts)), float(np.min(ts))
+
+
+# ----------------------------------------------------------------------------- config 3
+def make_cfg3(dev, seed=3):
+    """8 sequences, L ~ U{1024..8192} (not rounded to the block), packed; q/k contiguous as after
+    RoPE, v a strided view of the fused projection output (row stride 4096), random page tables,
+    last 32 tokens of each sequence uncommitted (slot -1) as in the engine's prefill."""
+    import oracle
+    g = torch.Generator().manual_seed(seed)
+    lens = [int(x) for x in torch.randint(1024, 8193, (8,), generator=g)]
+    N = sum(lens)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    fused = torch.empty(N, (HQ + 2 * HKV) * D, dtype=torch.bfloat16)
+    for s in range(0, N, 4096):                      # chunked: keeps host memory flat
+        fused[s:s + 4096] = torch.randn(min(4096, N - s), fused.shape[1], generator=g).bfloat16()
+    n_pages = sum((L + PAGE - 1) // PAGE for L in lens) + 64
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    slots = []
+    for L in lens:
+        n = (L + PAGE - 1) // PAGE
+        table, perm = perm[:n], perm[n:]
+        slots += oracle.get_slots(table, 0, L - S) + [-1] * S
+    host = dict(lens=lens, cu=cu, fused=fused, slots=torch.tensor(slots, dtype=torch.int32), n_pages=n_pages)
+    dfused = fused.to(dev)
+    gpu = dict(
+        q=dfused[:, :HQ * D].reshape(N, HQ, D).contiguous(),
+        k=dfused[:, HQ * D:(HQ + HKV) * D].reshape(N, HKV, D).contiguous(),
+        v=dfused[:, (HQ + HKV) * D:].view(N, HKV, D),
+        cu=cu.to(dev), slots=host["slots"].to(dev),
+        k_cache=torch.zeros(n_pages, PAGE, HKV, D, dtype=torch.bfloat16, device=dev),
+        v_cache=torch.zeros(n_pages, PAGE, HKV, D, dtype=torch.bfloat16, device=dev),
+    )
+    return host, gpu
+
+
+def cfg3_work(lens):
+    import oracle
+    pairs = sum(oracle.staircase_pairs(L, S) for L in lens)
+    stored = sum(L - S for L in lens)
+    return dict(pairs=pairs, flops=4 * D * HQ * pairs, store_bytes=2 * 2 * HKV * D * 2 * stored, tokens=sum(lens))
+
+
+# ----------------------------------------------------------------------------- config 2
+def make_cfg2(dev, n_sets=4, seed=2):
+    """16 sequences, prefix U{512..4096} + 32, page 256, page tables = disjoint slices of a random
+    permutation of a 64k-page pool (2 x 32 GiB, only the referenced pages are filled).  n_sets
+    independent page sets are rotated so the 256 MB last-level cache does not hold the K/V."""
+    g = torch.Generator().manual_seed(seed)
+    bs, pool = 16, 65536
+    ctxs = [int(x) + S for x in torch.randint(512, 4097, (bs,), generator=g)]
+    maxp = max((c + PAGE - 1) // PAGE for c in ctxs)
+    k_cache = torch.empty(pool, PAGE, HKV, D, dtype=torch.bfloat16, device=dev)
+    v_cache = torch.empty(pool, PAGE, HKV, D, dtype=torch.bfloat16, device=dev)
+    perm = torch.randperm(pool, generator=g)
+    at, sets = 0, []
+    for _ in range(n_sets):
+        bt = torch.full((bs, maxp), -1, dtype=torch.int32)
+        for b, c in enumerate(ctxs):
+            n = (c + PAGE - 1) // PAGE
+            bt[b, :n] = perm[at:at + n].to(torch.int32)
+            at += n
+        ids = bt[bt >= 0].long().to(dev)
+        k_cache[ids] = torch.randn(ids.numel(), PAGE, HKV, D, device=dev, dtype=torch.float32).bfloat16()
+        v_cache[ids] = torch.randn(ids.numel(), PAGE, HKV, D, device=dev, dtype=torch.float32).bfloat16()
+        sets.append(bt.to(dev))
+    q = torch.randn(bs, S, HQ, D, generator=g).bfloat16().to(dev)
+    lens = torch.tensor(ctxs, dtype=torch.int32, device=dev)
+    sum_ctx = sum(ctxs)
+    work = dict(flops=4 * D * HQ * S * sum_ctx, bytes=2 * HKV * D * 2 * sum_ctx + 2 * bs * S * HQ * D * 2, sum_ctx=sum_ctx)
+    return dict(q=q, k_cache=k_cache, v_cache=v_cache, tables=sets, lens=lens, ctxs=ctxs, work=work)
+
+
+# ----------------------------------------------------------------------------- config 4
+def make_cfg4(dev, n_sets=2, seed=4):
+    """[32 x 32 x 151936] bf16 logits ~ N(0, 3^2), 50-100 % of each block masked; two logits
+    buffers are rotated (622 MB > last-level cache)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    gc = torch.Generator().manual_seed(seed)
+    sets = []
+    for _ in range(n_sets):
+        logits = torch.empty(32, S, VOCAB, dtype=torch.bfloat16, device=dev)
+        for b in range(32):
+            logits[b] = (torch.randn(S, VOCAB, generator=g, device=dev) * 3).bfloat16()
+        sets.append(logits)
+    tokens = torch.randint(0, 1000, (32, S), generator=gc, dtype=torch.int64)
+    for b in range(32):
+        n = int(torch.randint(S // 2, S + 1, (1,), generator=gc))
+        tokens[b, torch.randperm(S, generator=gc)[:n]] = MASK_ID
+    return dict(logits=sets, tokens=tokens, bytes=32 * S * VOCAB * 2)
+
+
+# ----------------------------------------------------------------------------- CPU baseline
+def cpu_baseline(host3):
+    """The oracle on the host cores, bounded: one config-3 sequence of 4096 tokens through SDPA
+    with the explicit [L, L] staircase mask (bf16 inputs upcast to fp32), timed 3 times."""
+    import oracle
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    L = 4096
+    fused = host3["fused"][:L]
+    q = fused[:, :HQ * D].reshape(L, HQ, D)
+    k = fused[:, HQ * D:(HQ + HKV) * D].reshape(L, HKV, D)
+    v = fused[:, (HQ + HKV) * D:].reshape(L, HKV, D)
+    cu = [0, L]
+    oracle.staircase_attn_varlen(q[:512], k[:512], v[:512], [0, 512], S)      # warm-up
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        oracle.staircase_attn_varlen(q, k, v, cu, S)
+        ts.append(time.perf_counter() - t0)
+    flops = 4 * D * HQ * oracle.staircase_pairs(L, S)
+    t = float(np.median(ts))
+    return dict(value=round(flops / t / 1e12, 5), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"oracle (torch SDPA fp32 + explicit boolean staircase mask) on one sequence of {L} tokens "
+                       f"of the config-3 input, median of 3 runs, {t * 1e3:.0f} ms each; flops counted on visible pairs only",
+                ms=round(t * 1e3, 2))
+
+
+def cpu_side_ops(host3, cfg4_tokens):
+    """Bounded CPU timings of the two bandwidth ops, reported next to their GPU numbers."""
+    import oracle
+    out = {}
+    N = 4096
+    fused = host3["fused"][:N]
+    k = fused[:, HQ * D:(HQ + HKV) * D].reshape(N, HKV * D)
+    v = fused[:, (HQ + HKV) * D:].reshape(N, HKV * D).contiguous()
+    kc = torch.zeros(N + 512, HKV * D, dtype=torch.bfloat16)
+    vc = torch.zeros_like(kc)
+    idx = torch.randperm(N + 512)[:N]
+    t0 = time.perf_counter()
+    for _ in range(5):
+        kc.index_copy_(0, idx, k)
+        vc.index_copy_(0, idx, v)
+    t = (time.perf_counter() - t0) / 5
+    out["store_kvcache"] = dict(value=round(N * 2 * 2 * HKV * D * 2 / t / 1e9, 3), unit="GB/s",
+                                sample=f"index_copy_ of {N} rows, 5 runs")
+    g = torch.Generator().manual_seed(0)
+    rows = (torch.randn(64, VOCAB, generator=g) * 3).bfloat16()
+    t0 = time.perf_counter()
+    x0, p = oracle.confidence_argmax(rows.float().numpy()[None])
+    t = time.perf_counter() - t0
+    out["unmask"] = dict(value=round(rows.numel() * 2 / t / 1e9, 3), unit="GB/s", sample="oracle softmax+argmax on 64 rows")
+    return out
+
+
+# ----------------------------------------------------------------------------- main
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: step,store,paged,unmask (default all)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import mdx
+    if not mdx.library_path().exists():
+        sys.exit("bench.py: libmdx.so is missing; build it first (python mineru-diffusion_amd/build.py)")
+    only = set(filter(None, args.only.split(",")))
+    want = lambda leg: not only or leg in only      # noqa: E731
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    K, W = args.steps, args.warmup
+    result_ops = {}
+
+    # ---------------- config 3: the step (store + staircase attention) -----------------------------
+    log("[bench] building config 3 inputs")
+    host3, g3 = make_cfg3(dev)
+    work3 = cfg3_work(host3["lens"])
+    max_len = max(host3["lens"])
+    attn = mdx.Attention(HQ, D, 1 / math.sqrt(D), HKV)
+    attn.k_cache, attn.v_cache = g3["k_cache"], g3["v_cache"]
+    mdx.set_context(True, g3["cu"], g3["cu"], max_len, max_len, g3["slots"], None, None, block_size=S)
+
+    def attn_only(_):
+        return mdx.sparse_attn_varlen(g3["q"], g3["k"], g3["v"], g3["cu"], g3["cu"], S, max_seqlen=max_len)
+
+    def store_only(_):
+        mdx.store_kvcache(g3["k"], g3["v"], g3["k_cache"], g3["v_cache"], g3["slots"])
+
+    ms_step = attn_ms = float("nan")
+    if want("step"):
+        log("[bench] timing the step")
+        for _ in range(W):
+            attn(g3["q"], g3["k"], g3["v"])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            attn(g3["q"], g3["k"], g3["v"])
+        torch.cuda.synchronize()
+        ms_step = (time.perf_counter() - t0) * 1e3 / K
+        attn_ms, attn_min = time_kernel(attn_only, 2, K)
+        result_ops["staircase_attn"] = dict(
+            ms=round(attn_ms, 4), ms_min=round(attn_min, 4), tflops=round(work3["flops"] / attn_ms / 1e9, 2),
+            roofline=dict(bound="mfma", achieved=round(work3["flops"] / attn_ms / 1e9, 2), peak=PEAK_MFMA_TFLOPS,
+                          unit="TFLOP/s", frac=round(work3["flops"] / attn_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), traffic=None))
+    if want("store"):
+        st_ms, st_min = time_kernel(store_only, W, K)
+        gbs = work3["store_bytes"] / st_ms / 1e6
+        result_ops["store_kvcache"] = dict(
+            ms=round(st_ms, 4), ms_min=round(st_min, 4),
+            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+    mdx.reset_context()
+
+    # ---------------- config 2: paged single-block attention ---------------------------------------
+    if want("paged"):
+        log("[bench] building config 2 inputs (64 GiB page pool, referenced pages only are filled)")
+        c2 = make_cfg2(dev)
+
+        def paged(i):
+            return mdx.flash_attn_with_kvcache(c2["q"], c2["k_cache"], c2["v_cache"], cache_seqlens=c2["lens"],
+                                               block_table=c2["tables"][i % len(c2["tables"])],
+                                               softmax_scale=1 / math.sqrt(D), causal=False)
+        pg_ms, pg_min = time_kernel(paged, W, K)
+        gbs = c2["work"]["bytes"] / pg_ms / 1e6
+        result_ops["paged_block_attn"] = dict(
+            ms=round(pg_ms, 4), ms_min=round(pg_min, 4), tflops=round(c2["work"]["flops"] / pg_ms / 1e9, 2),
+            mfma_frac=round(c2["work"]["flops"] / pg_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), sum_ctx=c2["work"]["sum_ctx"],
+            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        del c2
+        torch.cuda.empty_cache()
+
+    # ---------------- config 4: unmask step -----------------------------------------------------------
+    cfg4_tokens = None
+    if want("unmask"):
+        log("[bench] building config 4 inputs")
+        c4 = make_cfg4(dev)
+        cfg4_tokens = c4["tokens"]
+        dtok = [c4["tokens"].clone().to(dev) for _ in range(K + W + 1)]
+        state = {"i": 0}
+
+        def unmask(i):
+            t = dtok[state["i"] % len(dtok)]
+            state["i"] += 1
+            return mdx.unmask_step(c4["logits"][i % len(c4["logits"])], t, MASK_ID, 0.9, 4)
+        um_ms, um_min = time_kernel(unmask, W, K)
+        gbs = c4["bytes"] / um_ms / 1e6
+        result_ops["unmask_step"] = dict(
+            ms=round(um_ms, 4), ms_min=round(um_min, 4),
+            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        del c4, dtok
+        torch.cuda.empty_cache()
+
+    # ---------------- CPU baseline (bounded) -------------------------------------------------------------
+    cpu = None
+    if not args.skip_cpu:
+        log("[bench] CPU baseline (oracle on host cores)")
+        cpu = cpu_baseline(host3)
+        try:
+            cpu["other_ops"] = cpu_side_ops(host3, cfg4_tokens)
+        except Exception as e:  # the side numbers are informative only
+            cpu["other_ops"] = {"error": str(e)}
+
+    value = work3["flops"] / ms_step / 1e9 if ms_step == ms_step else None
+    line = {
+        "metric": "staircase-attn TFLOP/s (%MFMA peak) + block-diffusion decode tokens/s, 1 GPU",
+        "value": None if value is None else round(value, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": None if value is None else round(ms_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "config 3: one prefill pass of the attention layer (store_kvcache + staircase "
+                               "block-prefill attention) over 8 packed sequences",
+                   "seq_lens": host3["lens"], "total_tokens": work3["tokens"], "block": S, "num_q_heads": HQ,
+                   "num_kv_heads": HKV, "head_dim": D, "page_size": PAGE, "visible_pairs": work3["pairs"],
+                   "algorithmic_gflop": round(work3["flops"] / 1e9, 2)},
+        "roofline": result_ops.get("staircase_attn", {}).get("roofline"),
+        "cpu_baseline": cpu,
+        "ops": result_ops,
+        "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
