@@ -39,7 +39,6 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 constexpr int kHeadDim = 128;
 constexpr int kRowBytes = kHeadDim * 2;      // one K or V row of one head
 constexpr int kLdsPitch = kRowBytes + 16;    // 272: consecutive rows shift by 4 banks
-constexpr int kThreads = 256;                // 4 wavefronts per workgroup
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kMinusBig = -1.0e30f;        // finite initial running max (avoids inf - inf)
 
@@ -203,20 +202,22 @@ __device__ __forceinline__ void load_q(bf16x8 (&q)[8], const __bf16* q_row, int 
     }
 }
 
-// Global -> register staging of one K/V tile of TK rows x 256 B by 256 threads:
-// thread t moves chunk t%16 (16 B) of rows t/16, t/16+16, ...
-template <int TK>
+// Global -> register staging of one K/V tile of TK rows x 256 B by T threads:
+// thread t moves chunk t%16 (16 B) of rows t/16, t/16 + T/16, ...
+template <int TK, int T>
 struct TileRegs {
-    u32x4 k[TK / 16];
-    u32x4 v[TK / 16];
+    static constexpr int kPasses = TK * 16 / T;
+    static_assert(kPasses >= 1 && (TK * 16) % T == 0, "tile does not divide over the workgroup");
+    u32x4 k[kPasses];
+    u32x4 v[kPasses];
 };
 
-template <int TK>
-__device__ __forceinline__ void store_tile(char* lds_k, char* lds_v, const TileRegs<TK>& regs, int tid) {
+template <int TK, int T>
+__device__ __forceinline__ void store_tile(char* lds_k, char* lds_v, const TileRegs<TK, T>& regs, int tid) {
     const int chunk = tid & 15, row0 = tid >> 4;
 #pragma unroll
-    for (int p = 0; p < TK / 16; ++p) {
-        const int off = (row0 + 16 * p) * kLdsPitch + chunk * 16;
+    for (int p = 0; p < TileRegs<TK, T>::kPasses; ++p) {
+        const int off = (row0 + (T / 16) * p) * kLdsPitch + chunk * 16;
         *reinterpret_cast<u32x4*>(lds_k + off) = regs.k[p];
         *reinterpret_cast<u32x4*>(lds_v + off) = regs.v[p];
     }

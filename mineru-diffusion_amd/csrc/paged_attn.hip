@@ -27,6 +27,7 @@ using namespace mdx_attn;
 
 constexpr int kTileKeys = 128;     // 4 wavefronts x 32 keys
 constexpr int kMaxSq = 32;
+constexpr int kThreads = 256;
 
 struct PagedParams {
     const __bf16* q; __bf16* o; const __bf16* k_cache; const __bf16* v_cache;
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedP
     const int32_t* bt = P.block_table + (int64_t)b * P.bt_stride;
     const int chunk = tid & 15, trow = tid >> 4;
     const int n_tiles = (key_end - key_begin + kTileKeys - 1) / kTileKeys;
-    TileRegs<kTileKeys> regs;
+    TileRegs<kTileKeys, 256> regs;
     // A tile never straddles a page (page_size % kTileKeys == 0, key_begin % kTileKeys == 0).
     auto fetch = [&](int t) {
         const int key0 = key_begin + t * kTileKeys;
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedP
     bool cur_ok = fetch(0);
     for (int t = 0; t < n_tiles; ++t) {
         __syncthreads();
-        store_tile<kTileKeys>(lds_k, lds_v, regs, tid);
+        store_tile<kTileKeys, 256>(lds_k, lds_v, regs, tid);
         __syncthreads();
         const bool this_ok = cur_ok;
         if (t + 1 < n_tiles) cur_ok = fetch(t + 1);

@@ -7,15 +7,18 @@
 //
 // Work decomposition (not the reference's one-program-per-(sequence, head)):
 // everything is indexed in PADDED coordinates ip = i + pad, jp = j + pad, in
-// which block boundaries fall on multiples of S.  A workgroup of 4 wavefronts
-// owns 128 consecutive padded query rows of one sequence and one group of NH
-// query heads sharing a KV head; wavefront w owns rows 32w..32w+31.  For
-// S >= 32 every 32-row tile lies inside one block, so all its rows share one
-// key limit and no element of the tile interior is ever masked: only the very
-// first keys (jp < pad) and, for S < 32, the tiles straddling the limit take
-// the masked path.  K/V tiles of 64 keys are staged once per workgroup in LDS
-// (global -> registers one tile ahead -> LDS) and reused by all 4 wavefronts
-// and by the NH heads of the GQA group.
+// which block boundaries fall on multiples of S.  A wavefront owns 32
+// consecutive padded query rows of ONE query head.  A workgroup of 8
+// wavefronts owns NBLK such row tiles for each of HPW query heads that share
+// a KV head (HPW = 2, NBLK = 4 for grouped-query attention: 128 rows x 2
+// heads; HPW = 1, NBLK = 8 otherwise), so the K/V tiles it stages in LDS are
+// shared by all 8 wavefronts.  Two wavefronts live on every SIMD, which lets
+// the hardware overlap one wavefront's MFMAs with the other's softmax.
+// For S >= 32 every 32-row tile lies inside one block, so all its rows share
+// one key limit and no element of the tile interior is ever masked: only the
+// very first keys (jp < pad) and, for S < 32, the tiles straddling the limit
+// take the masked path.  K/V tiles of 64 keys are double-buffered in LDS
+// (global -> registers one tile ahead -> LDS), one barrier per tile.
 //
 // Launch order: workgroups are numbered heaviest-first (last row group of every
 // sequence first), and the head group is the fastest-varying index so that
@@ -29,7 +32,8 @@ namespace {
 using namespace mdx_attn;
 
 constexpr int kTileKeys = 64;      // keys staged in LDS per iteration
-constexpr int kRowsPerWg = 128;    // 4 wavefronts x 32 query rows
+constexpr int kThreads = 512;      // 8 wavefronts
+constexpr int kTileBytes = kTileKeys * kLdsPitch;
 
 struct StaircaseParams {
     const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o;
@@ -40,11 +44,12 @@ struct StaircaseParams {
     float c;                                                   // scale * log2(e)
 };
 
-template <int NH>
+template <int HPW, int NBLK>
 __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const StaircaseParams P)
 {
-    __shared__ __attribute__((aligned(16))) char lds_k[kTileKeys * kLdsPitch];
-    __shared__ __attribute__((aligned(16))) char lds_v[kTileKeys * kLdsPitch];
+    static_assert(HPW * NBLK * 64 == kThreads, "8 wavefronts per workgroup");
+    constexpr int kRowsPerWg = 32 * NBLK;
+    __shared__ __attribute__((aligned(16))) char lds[2][2 * kTileBytes];   // [buffer][K tile, V tile]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
@@ -64,18 +69,16 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     const int row_g0 = rg * kRowsPerWg;                        // first padded row of the workgroup
     if (row_g0 >= Lp) return;
 
-    const int head0 = hg * NH;
-    const int kvh = head0 / P.heads_per_kv;
+    const int head = hg * HPW + wave / NBLK;                   // this wavefront's query head
+    const int kvh = (hg * HPW) / P.heads_per_kv;               // all heads of the workgroup share it
 
     // ---- this wavefront's 32 rows ----
-    const int row_w0 = row_g0 + wave * 32;
+    const int row_w0 = row_g0 + (wave % NBLK) * 32;
     const int ip = row_w0 + r;                                 // this lane's padded query row
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
-    bf16x8 q[NH][8];
-#pragma unroll
-    for (int h = 0; h < NH; ++h)
-        load_q(q[h], row_ok ? P.q + tok * P.q_st + (int64_t)(head0 + h) * P.q_sh : nullptr, H);
+    bf16x8 q[1][8];
+    load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
 
     // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
@@ -85,24 +88,23 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
     const int n_tiles = (wg_hi + kTileKeys - 1) / kTileKeys;
 
-    WaveState<NH> st;
+    WaveState<1> st;
     st.init();
 
-    // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t ----
+    // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t (other buffer: t-1) ----
     const __bf16* kbase = P.k + (int64_t)kvh * P.k_sh;
     const __bf16* vbase = P.v + (int64_t)kvh * P.v_sh;
     const int chunk = tid & 15, trow = tid >> 4;
-    TileRegs<kTileKeys> regs;
+    TileRegs<kTileKeys, kThreads> regs;
     auto fetch = [&](int t) {
 #pragma unroll
-        for (int p = 0; p < kTileKeys / 16; ++p) {
-            const int jp = t * kTileKeys + trow + 16 * p;
-            const bool ok = jp >= pad && jp < Lp;
-            if (ok) {
+        for (int p = 0; p < TileRegs<kTileKeys, kThreads>::kPasses; ++p) {
+            const int jp = t * kTileKeys + trow + (kThreads / 16) * p;
+            if (jp >= pad && jp < Lp) {
                 const int64_t kt = (int64_t)seq0 + (jp - pad);
                 regs.k[p] = *reinterpret_cast<const u32x4*>(kbase + kt * P.k_st + chunk * 8);
                 regs.v[p] = *reinterpret_cast<const u32x4*>(vbase + kt * P.v_st + chunk * 8);
-            } else {
+            } else {                           // keys outside the sequence: zero rows, masked below
                 regs.k[p] = u32x4{0, 0, 0, 0};
                 regs.v[p] = u32x4{0, 0, 0, 0};
             }
@@ -110,42 +112,47 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     };
 
     fetch(0);
+    store_tile<kTileKeys, kThreads>(lds[0], lds[0] + kTileBytes, regs, tid);
+    if (n_tiles > 1) fetch(1);
+    __syncthreads();
     for (int t = 0; t < n_tiles; ++t) {
-        __syncthreads();                       // everyone is done reading the previous tile
-        store_tile<kTileKeys>(lds_k, lds_v, regs, tid);
-        __syncthreads();
-        if (t + 1 < n_tiles) fetch(t + 1);     // in flight while this tile is consumed
-
+        const char* lds_k = lds[t & 1];
+        const char* lds_v = lds_k + kTileBytes;
         const int key0 = t * kTileKeys;
         if (key0 < wave_hi) {
-            const bool full = key0 >= pad && key0 + kTileKeys <= wave_hi_min;
-            if (full) {
-                attn_step<NH, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+            if (key0 >= pad && key0 + kTileKeys <= wave_hi_min) {
+                attn_step<1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else if (key0 + 32 < wave_hi) {
-                attn_step<NH, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+            } else if (key0 >= pad && key0 + 32 <= wave_hi_min) {
+                attn_step<1, 1, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else {
-                attn_step<NH, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             }
         }
+        if (t + 1 < n_tiles) {
+            // the other buffer was last read in iteration t-1, which every wavefront has left
+            char* nk = lds[(t + 1) & 1];
+            store_tile<kTileKeys, kThreads>(nk, nk + kTileBytes, regs, tid);
+            if (t + 2 < n_tiles) fetch(t + 2);
+        }
+        __syncthreads();
     }
 
     // ---- epilogue: O = O^T / l, bf16, 4 consecutive d per store ----
     if (!row_ok) return;
+    const float inv = 1.0f / both_halves_sum(st.l[0]);
+    __bf16* orow = P.o + tok * P.o_st + (int64_t)head * P.o_sh;
 #pragma unroll
-    for (int h = 0; h < NH; ++h) {
-        const float inv = 1.0f / both_halves_sum(st.l[h]);
-        __bf16* orow = P.o + tok * P.o_st + (int64_t)(head0 + h) * P.o_sh;
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int g = 0; g < 4; ++g) {
+            typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+            bf16x4 out;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-                bf16x4 out;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[h][dt][4 * g + e] * inv);
-                *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
-            }
-    }
+            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
+            *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+        }
 }
 
 }  // namespace
@@ -181,7 +188,8 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                 MDX_EUNSUPPORTED, "staircase_attn: q/k/v/o must be 16-byte aligned with strides that are multiples of 8 elements");
 
     const int G = num_q_heads / num_kv_heads;
-    const int NH = (G % 2 == 0) ? 2 : 1;
+    const int HPW = (G % 2 == 0) ? 2 : 1;          // query heads per workgroup (they share a KV head)
+    const int rows_per_wg = 32 * (8 / HPW);
     StaircaseParams P;
     P.q = (const __bf16*)q; P.k = (const __bf16*)k; P.v = (const __bf16*)v; P.o = (__bf16*)o;
     P.q_st = q_stride_t; P.q_sh = q_stride_h; P.k_st = k_stride_t; P.k_sh = k_stride_h;
@@ -189,14 +197,14 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.cu_seqlens = cu_seqlens_k;
     P.batch = batch;
     const int64_t max_l = max_seqlen < total_tokens ? max_seqlen : total_tokens;
-    P.n_row_groups = (int)((max_l + staircase_size - 1 + kRowsPerWg - 1) / kRowsPerWg);
-    P.n_head_groups = num_q_heads / NH;
+    P.n_row_groups = (int)((max_l + staircase_size - 1 + rows_per_wg - 1) / rows_per_wg);
+    P.n_head_groups = num_q_heads / HPW;
     P.heads_per_kv = G;
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
     const int64_t grid = (int64_t)P.n_row_groups * batch * P.n_head_groups;
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
-    if (NH == 2) staircase_attn_kernel<2><<<(unsigned)grid, kThreads, 0, stream>>>(P);
-    else         staircase_attn_kernel<1><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    if (HPW == 2) staircase_attn_kernel<2, 4><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    else          staircase_attn_kernel<1, 8><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     return mdx::check_launch("staircase_attn");
 }
