@@ -54,11 +54,47 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
 
-    // workgroup -> (head group, sequence, row group), heaviest row groups first
-    int id = blockIdx.x;
-    const int hg = id % P.n_head_groups; id /= P.n_head_groups;
-    const int b = id % P.batch;          id /= P.batch;
-    const int rg = P.n_row_groups - 1 - id;
+    // ---- workgroup -> (head group, sequence b, row group rg) -----------------------------------
+    // Row groups are handed out heaviest-first (the last row group of a sequence attends to the
+    // most keys).  The dispatcher deals consecutive workgroups round-robin to XCDs and shader
+    // engines and blocks on a full one, so neighbours in launch order must weigh the same:
+    // the head group varies fastest, then the sequences that own a row group at this level, and
+    // workgroups that find no work may only sit at the very end of the grid.  With up to 64
+    // sequences each wavefront derives this dense numbering itself (lane b holds sequence b's
+    // row-group count, lane r evaluates F(r) = #pairs at level >= r); beyond that the grid is the
+    // full (level x sequence) rectangle and absent pairs return at once.
+    const int hg = blockIdx.x % P.n_head_groups;
+    const int j = blockIdx.x / P.n_head_groups;
+    int b, rg;
+    if (P.batch <= 64) {
+        int g = 0;                                             // row groups of sequence `lane`
+        if (lane < P.batch) {
+            const int len = P.cu_seqlens[lane + 1] - P.cu_seqlens[lane];
+            if (len > 0) g = ((((len + (1 << P.log2_s) - 1) >> P.log2_s) << P.log2_s) + kRowsPerWg - 1) / kRowsPerWg;
+        }
+        int level = -1, f_level = 0;
+        for (int base = 0; base < P.n_row_groups; base += 64) {
+            const int r_lane = base + lane;
+            int f = 0;
+            for (int s = 0; s < P.batch; ++s) f += max(0, __builtin_amdgcn_readlane(g, s) - r_lane);
+            const unsigned long long above = __ballot(f > j);  // F decreases with the level: low lanes
+            if (above == 0) break;
+            const int n = __popcll(above);
+            level = base + n - 1;
+            f_level = __builtin_amdgcn_readlane(f, n - 1);
+            if (n < 64) break;
+        }
+        if (level < 0) return;                                 // past the last pair
+        const unsigned long long owners = __ballot(g > level); // sequences that have this row group
+        const int nth = j - f_level + __popcll(owners);        // index among them
+        const int before = __popcll(owners & ((1ull << lane) - 1ull));
+        const unsigned long long hit = __ballot(((owners >> lane) & 1ull) != 0 && before == nth);
+        b = __ffsll((long long)hit) - 1;
+        rg = level;
+    } else {
+        b = j % P.batch;
+        rg = P.n_row_groups - 1 - j / P.batch;
+    }
 
     const int seq0 = P.cu_seqlens[b];
     const int L = P.cu_seqlens[b + 1] - seq0;
@@ -202,7 +238,10 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.heads_per_kv = G;
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
-    const int64_t grid = (int64_t)P.n_row_groups * batch * P.n_head_groups;
+    // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence
+    const int64_t n_pairs = batch <= 64 ? (total_tokens + (int64_t)batch * (staircase_size + rows_per_wg - 2)) / rows_per_wg
+                                        : (int64_t)P.n_row_groups * batch;
+    const int64_t grid = n_pairs * P.n_head_groups;
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
     if (HPW == 2) staircase_attn_kernel<2, 4><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     else          staircase_attn_kernel<1, 8><<<(unsigned)grid, kThreads, 0, stream>>>(P);
