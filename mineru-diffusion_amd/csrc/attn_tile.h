@@ -41,6 +41,7 @@ constexpr int kRowBytes = kHeadDim * 2;      // one K or V row of one head
 constexpr int kLdsPitch = kRowBytes + 16;    // 272: consecutive rows shift by 4 banks
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kMinusBig = -1.0e30f;        // finite initial running max (avoids inf - inf)
+constexpr float kMaxSlack = 8.0f;            // running max may lag by up to 2^8 before O is rescaled
 
 __device__ __forceinline__ int key_of_reg(int i, int H) {
     return 16 * (i >> 3) + 4 * (i & 3) + 2 * H + ((i >> 2) & 1);
@@ -140,8 +141,13 @@ __device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, 
 #pragma unroll
             for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[h][u][i]);
         mx = other_half_max(mx);
-        const float m_new = fmaxf(st.m[h], mx * c);
-        const float alpha = __builtin_amdgcn_exp2f(st.m[h] - m_new);
+        // Lazy rescale: the running max only moves when some query's new max exceeds it by more
+        // than kMaxSlack (log2 units).  Until then probabilities are taken relative to the stale
+        // max (at most 2^kMaxSlack, harmless in fp32/bf16) and O, l need no rescaling; the final
+        // O / l is unchanged because numerator and denominator share the same reference.
+        const float m_cand = fmaxf(st.m[h], mx * c);
+        const bool moved = __any(m_cand > st.m[h] + kMaxSlack);        // wave-uniform
+        const float m_new = moved ? m_cand : st.m[h];
         float sum = 0.f;
 #pragma unroll
         for (int u = 0; u < NSUB; ++u)
@@ -153,14 +159,16 @@ __device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, 
                     sum += e;
                     p[h][u][t][j] = (__bf16)e;
                 }
-        st.l[h] = st.l[h] * alpha + sum;
-        st.m[h] = m_new;
-        if (__any(alpha != 1.0f)) {          // wave-uniform: skip the rescale when no query's max moved
+        if (moved) {
+            const float alpha = __builtin_amdgcn_exp2f(st.m[h] - m_new);
+            st.l[h] *= alpha;
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) st.o[h][t][i] *= alpha;
+            st.m[h] = m_new;
         }
+        st.l[h] += sum;
     }
 
     // ---- O^T += V^T P^T ------------------------------------------------------

@@ -128,23 +128,31 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     st.init();
 
     // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t (other buffer: t-1) ----
-    const __bf16* kbase = P.k + (int64_t)kvh * P.k_sh;
-    const __bf16* vbase = P.v + (int64_t)kvh * P.v_sh;
+    // Thread-private row pointers walk down the sequence one tile per fetch; rows outside the
+    // sequence (only possible in the first and last tiles) are never dereferenced.
     const int chunk = tid & 15, trow = tid >> 4;
+    constexpr int kPasses = TileRegs<kTileKeys, kThreads>::kPasses;
+    constexpr int kRowsPerPass = kThreads / 16;
+    const int64_t row0 = (int64_t)seq0 - pad + trow;          // token of LDS row `trow` of tile 0
+    const __bf16* kcur = P.k + (int64_t)kvh * P.k_sh + row0 * P.k_st + chunk * 8;
+    const __bf16* vcur = P.v + (int64_t)kvh * P.v_sh + row0 * P.v_st + chunk * 8;
+    const int64_t k_pass = (int64_t)kRowsPerPass * P.k_st, v_pass = (int64_t)kRowsPerPass * P.v_st;
     TileRegs<kTileKeys, kThreads> regs;
-    auto fetch = [&](int t) {
+    auto fetch = [&](int t) {                  // called with t = 0, 1, 2, ... in order
+        const bool interior = t * kTileKeys >= pad && (t + 1) * kTileKeys <= Lp;   // uniform
 #pragma unroll
-        for (int p = 0; p < TileRegs<kTileKeys, kThreads>::kPasses; ++p) {
-            const int jp = t * kTileKeys + trow + (kThreads / 16) * p;
-            if (jp >= pad && jp < Lp) {
-                const int64_t kt = (int64_t)seq0 + (jp - pad);
-                regs.k[p] = *reinterpret_cast<const u32x4*>(kbase + kt * P.k_st + chunk * 8);
-                regs.v[p] = *reinterpret_cast<const u32x4*>(vbase + kt * P.v_st + chunk * 8);
+        for (int p = 0; p < kPasses; ++p) {
+            const int jp = t * kTileKeys + trow + kRowsPerPass * p;
+            if (interior || (jp >= pad && jp < Lp)) {
+                regs.k[p] = *reinterpret_cast<const u32x4*>(kcur + p * k_pass);
+                regs.v[p] = *reinterpret_cast<const u32x4*>(vcur + p * v_pass);
             } else {                           // keys outside the sequence: zero rows, masked below
                 regs.k[p] = u32x4{0, 0, 0, 0};
                 regs.v[p] = u32x4{0, 0, 0, 0};
             }
         }
+        kcur += kPasses * k_pass;
+        vcur += kPasses * v_pass;
     };
 
     fetch(0);
