@@ -8,22 +8,22 @@
 // Work decomposition (not the reference's one-program-per-(sequence, head)):
 // everything is indexed in PADDED coordinates ip = i + pad, jp = j + pad, in
 // which block boundaries fall on multiples of S.  A wavefront owns 32
-// consecutive padded query rows of ONE query head.  A workgroup of 8
-// wavefronts owns NBLK such row tiles for each of HPW query heads that share
-// a KV head (HPW = 2, NBLK = 4 for grouped-query attention: 128 rows x 2
-// heads; HPW = 1, NBLK = 8 otherwise), so the K/V tiles it stages in LDS are
-// shared by all 8 wavefronts.  Two wavefronts live on every SIMD, which lets
-// the hardware overlap one wavefront's MFMAs with the other's softmax.
-// For S >= 32 every 32-row tile lies inside one block, so all its rows share
-// one key limit and no element of the tile interior is ever masked: only the
-// very first keys (jp < pad) and, for S < 32, the tiles straddling the limit
-// take the masked path.  K/V tiles of 64 keys are double-buffered in LDS
-// (global -> registers one tile ahead -> LDS), one barrier per tile.
+// consecutive padded query rows of one query head; a workgroup of 4 wavefronts
+// owns 128 consecutive rows of that head and stages the K/V tiles they share
+// in LDS.  Two such workgroups fit a CU (2 wavefronts per SIMD); they share no
+// barrier, so they drift out of phase and one's MFMAs overlap the other's
+// softmax arithmetic.  For S >= 32 every 32-row tile lies inside one block, so
+// all its rows share one key limit and no element of the tile interior is ever
+// masked: only the very first keys (jp < pad) and, for S < 32, the tiles
+// straddling the limit take the masked path.  K/V tiles of 64 keys are
+// double-buffered in LDS (global -> registers one tile ahead -> LDS), one
+// barrier per tile.
 //
 // Launch order: workgroups are numbered heaviest-first (last row group of every
-// sequence first), and the head group is the fastest-varying index so that
-// consecutive workgroups, which the dispatcher deals round-robin to the 8 XCDs,
-// keep one KV head's K/V stream per XCD L2 when there are 8 head groups.
+// sequence first); the query head varies fastest, ordered KV head first, so
+// that consecutive workgroups, which the dispatcher deals round-robin to the 8
+// XCDs, put all query heads of one KV head on the same XCD (one K/V stream per
+// XCD L2 when there are 8 KV heads).
 #include "mdx_common.h"
 #include "attn_tile.h"
 
@@ -32,24 +32,23 @@ namespace {
 using namespace mdx_attn;
 
 constexpr int kTileKeys = 64;      // keys staged in LDS per iteration
-constexpr int kThreads = 512;      // 8 wavefronts
+constexpr int kThreads = 256;      // 4 wavefronts, 2 workgroups per CU
+constexpr int kRowsPerWg = 128;    // 4 wavefronts x 32 query rows
 constexpr int kTileBytes = kTileKeys * kLdsPitch;
 
 struct StaircaseParams {
     const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o;
     int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;   // element strides: token, head
     const int32_t* cu_seqlens;
-    int batch, n_row_groups, n_head_groups, heads_per_kv;      // heads_per_kv = Hq / Hkv
+    int batch, n_row_groups, num_q_heads, num_kv_heads;
     int log2_s;
     float c;                                                   // scale * log2(e)
 };
 
-template <int HPW, int NBLK>
-__global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const StaircaseParams P)
+__global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const StaircaseParams P)
 {
-    static_assert(HPW * NBLK * 64 == kThreads, "8 wavefronts per workgroup");
-    constexpr int kRowsPerWg = 32 * NBLK;
-    __shared__ __attribute__((aligned(16))) char lds[2][2 * kTileBytes];   // [buffer][K tile, V tile]
+    __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
+    __shared__ __attribute__((aligned(16))) char lds_vbuf[2][kTileBytes];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
@@ -63,8 +62,8 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     // sequences each wavefront derives this dense numbering itself (lane b holds sequence b's
     // row-group count, lane r evaluates F(r) = #pairs at level >= r); beyond that the grid is the
     // full (level x sequence) rectangle and absent pairs return at once.
-    const int hg = blockIdx.x % P.n_head_groups;
-    const int j = blockIdx.x / P.n_head_groups;
+    const int hslot = blockIdx.x % P.num_q_heads;
+    const int j = blockIdx.x / P.num_q_heads;
     int b, rg;
     if (P.batch <= 64) {
         int g = 0;                                             // row groups of sequence `lane`
@@ -105,16 +104,16 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     const int row_g0 = rg * kRowsPerWg;                        // first padded row of the workgroup
     if (row_g0 >= Lp) return;
 
-    const int head = hg * HPW + wave / NBLK;                   // this wavefront's query head
-    const int kvh = (hg * HPW) / P.heads_per_kv;               // all heads of the workgroup share it
+    const int kvh = hslot % P.num_kv_heads;                    // launch order: KV head fastest
+    const int head = kvh * (P.num_q_heads / P.num_kv_heads) + hslot / P.num_kv_heads;
 
     // ---- this wavefront's 32 rows ----
-    const int row_w0 = row_g0 + (wave % NBLK) * 32;
+    const int row_w0 = row_g0 + wave * 32;
     const int ip = row_w0 + r;                                 // this lane's padded query row
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
-    bf16x8 q[1][8];
-    load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
+    bf16x8 q[8];
+    load_q(q, row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
 
     // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
@@ -124,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
     const int n_tiles = (wg_hi + kTileKeys - 1) / kTileKeys;
 
-    WaveState<1> st;
+    WaveState st;
     st.init();
 
     // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t (other buffer: t-1) ----
@@ -156,28 +155,25 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
     };
 
     fetch(0);
-    store_tile<kTileKeys, kThreads>(lds[0], lds[0] + kTileBytes, regs, tid);
+    store_tile<kTileKeys, kThreads>(lds_kbuf[0], lds_vbuf[0], regs, tid);
     if (n_tiles > 1) fetch(1);
     __syncthreads();
     for (int t = 0; t < n_tiles; ++t) {
-        const char* lds_k = lds[t & 1];
-        const char* lds_v = lds_k + kTileBytes;
+        const char* lds_k = lds_kbuf[t & 1];
+        const char* lds_v = lds_vbuf[t & 1];
         const int key0 = t * kTileKeys;
         if (key0 < wave_hi) {
             if (key0 >= pad && key0 + kTileKeys <= wave_hi_min) {
-                attn_step<1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else if (key0 + 32 < wave_hi) {
-                attn_step<1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
-            } else if (key0 >= pad && key0 + 32 <= wave_hi_min) {
-                attn_step<1, 1, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else {
-                attn_step<1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             }
         }
         if (t + 1 < n_tiles) {
             // the other buffer was last read in iteration t-1, which every wavefront has left
-            char* nk = lds[(t + 1) & 1];
-            store_tile<kTileKeys, kThreads>(nk, nk + kTileBytes, regs, tid);
+            store_tile<kTileKeys, kThreads>(lds_kbuf[(t + 1) & 1], lds_vbuf[(t + 1) & 1], regs, tid);
             if (t + 2 < n_tiles) fetch(t + 2);
         }
         __syncthreads();
@@ -185,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
 
     // ---- epilogue: O = O^T / l, bf16, 4 consecutive d per store ----
     if (!row_ok) return;
-    const float inv = 1.0f / both_halves_sum(st.l[0]);
+    const float inv = 1.0f / both_halves_sum(st.l);
     __bf16* orow = P.o + tok * P.o_st + (int64_t)head * P.o_sh;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -194,7 +190,7 @@ __global__ __launch_bounds__(kThreads) void staircase_attn_kernel(const Staircas
             typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
             bf16x4 out;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
+            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[dt][4 * g + e] * inv);
             *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
         }
 }
@@ -231,9 +227,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                 v_stride_t % 8 == 0 && v_stride_h % 8 == 0 && o_stride_t % 4 == 0 && o_stride_h % 4 == 0,
                 MDX_EUNSUPPORTED, "staircase_attn: q/k/v/o must be 16-byte aligned with strides that are multiples of 8 elements");
 
-    const int G = num_q_heads / num_kv_heads;
-    const int HPW = (G % 2 == 0) ? 2 : 1;          // query heads per workgroup (they share a KV head)
-    const int rows_per_wg = 32 * (8 / HPW);
+    const int rows_per_wg = kRowsPerWg;
     StaircaseParams P;
     P.q = (const __bf16*)q; P.k = (const __bf16*)k; P.v = (const __bf16*)v; P.o = (__bf16*)o;
     P.q_st = q_stride_t; P.q_sh = q_stride_h; P.k_st = k_stride_t; P.k_sh = k_stride_h;
@@ -242,16 +236,15 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.batch = batch;
     const int64_t max_l = max_seqlen < total_tokens ? max_seqlen : total_tokens;
     P.n_row_groups = (int)((max_l + staircase_size - 1 + rows_per_wg - 1) / rows_per_wg);
-    P.n_head_groups = num_q_heads / HPW;
-    P.heads_per_kv = G;
+    P.num_q_heads = num_q_heads;
+    P.num_kv_heads = num_kv_heads;
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
     // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence
     const int64_t n_pairs = batch <= 64 ? (total_tokens + (int64_t)batch * (staircase_size + rows_per_wg - 2)) / rows_per_wg
                                         : (int64_t)P.n_row_groups * batch;
-    const int64_t grid = n_pairs * P.n_head_groups;
+    const int64_t grid = n_pairs * num_q_heads;
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
-    if (HPW == 2) staircase_attn_kernel<2, 4><<<(unsigned)grid, kThreads, 0, stream>>>(P);
-    else          staircase_attn_kernel<1, 8><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    staircase_attn_kernel<<<(unsigned)grid, kThreads, 0, stream>>>(P);
     return mdx::check_launch("staircase_attn");
 }
