@@ -7,17 +7,21 @@
 //
 // The op is HBM-bound (each K/V byte is used by only Sq * Hq/Hkv = 64 query
 // rows), so the design goal is to keep the whole chip streaming pages:
-//  * split-KV: workgroup (split, head group, sequence) owns `chunk` consecutive
-//    keys; there are far more workgroups than the bs*Hkv (sequence, KV head)
-//    pairs.  Splits past the context length exit at once.
-//  * a workgroup has 8 wavefronts, each owning 32 queries of ONE query head:
+//  * split-KV: a workgroup owns `chunk` consecutive keys of one sequence for
+//    one group of query heads; there are far more workgroups than the bs*Hkv
+//    (sequence, KV head) pairs.  Workgroups are numbered densely over the
+//    (sequence, split) pairs that exist (lane b of each wavefront holds the
+//    split count of sequence b), so the launch order has no holes: the
+//    dispatcher deals consecutive workgroups round-robin to XCDs and shader
+//    engines and stalls on a full one, which punishes interleaved no-op groups.
+//  * a workgroup has 4 wavefronts, each owning 32 queries of ONE query head:
 //    HPW heads that share a KV head (2 for grouped-query attention) times
-//    KW = 8/HPW key slices.  Every tile of 32*KW keys is staged in LDS by one
-//    pass of coalesced 16-byte loads and split between the key slices (32 keys
-//    per wavefront); the next tile's loads are in flight (in registers) while
-//    the current one is consumed.
-//  * the KW wavefront states of a head are merged through LDS (a tree), then
-//    either written as the final output (single split) or as an fp32 partial
+//    KW = 4/HPW key slices of 32 keys.  Two workgroups share a CU.
+//  * K/V tiles of 32*KW keys travel global -> registers -> LDS with 16-byte
+//    coalesced loads; two tiles are in flight in registers while a third is
+//    consumed from the double-buffered LDS, so HBM latency stays covered.
+//  * the KW wavefront states of a head are merged through LDS, then either
+//    written as the final output (single split) or as an fp32 partial
 //    (m, l, O) that a second, small kernel combines.
 #include "mdx_common.h"
 #include "attn_tile.h"
@@ -28,7 +32,7 @@ namespace {
 using namespace mdx_attn;
 
 constexpr int kMaxSq = 32;
-constexpr int kThreads = 512;      // 8 wavefronts
+constexpr int kThreads = 256;      // 4 wavefronts, 2 workgroups per CU
 constexpr int kChunkAlign = 256;   // split boundaries are multiples of this many keys
 
 struct PagedParams {
@@ -37,36 +41,54 @@ struct PagedParams {
     int64_t c_sp, c_st, c_sh;                       // cache strides: page, token, head
     const int32_t* block_table; int64_t bt_stride;
     const int32_t* context_lens;
-    int sq, heads_per_kv, page_size, max_pages;
+    int bs, sq, heads_per_kv, page_size, page_shift, max_pages;   // page_shift: log2(page_size) or -1
     int64_t num_pages;
-    int chunk, nsplit;                              // keys per split, splits per sequence (grid.x)
+    int chunk, nsplit;                              // keys per split, max splits per sequence
     int num_q_heads;
     float c;                                        // scale * log2(e)
     float* part_o; float* part_ml;                  // [bs, Hq, nsplit, 32, 128] and [bs, Hq, nsplit, 2, 32]
 };
 
-template <int HPW>
-__global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedParams P)
+template <int HPW, int DEPTH>
+__global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const PagedParams P)
 {
-    constexpr int KW = 8 / HPW;                     // key slices (wavefronts per head)
+    constexpr int KW = 4 / HPW;                     // key slices (wavefronts per head)
     constexpr int kTileKeys = 32 * KW;
     constexpr int kTileBytes = kTileKeys * kLdsPitch;
-    // K and V tiles; the region is reused for the cross-wavefront merge at the end.
-    __shared__ __attribute__((aligned(16))) char lds[2 * kTileBytes];
-    char* lds_k = lds;
-    char* lds_v = lds + kTileBytes;
+    constexpr int kPasses = TileRegs<kTileKeys, kThreads>::kPasses;   // 16 rows per pass
+    // [buffer][K tile, V tile]; the region is reused for the cross-wavefront merge at the end.
+    __shared__ __attribute__((aligned(16))) char lds[2][2 * kTileBytes];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
-    const int split = blockIdx.x, hg = blockIdx.y, b = blockIdx.z;
+    const int hg = blockIdx.x;
     const int kw = wave % KW;                       // this wavefront's key slice
     const int head = hg * HPW + wave / KW;          // and query head
 
+    // ---- workgroup -> (sequence b, split) ------------------------------------------------------
+    int b, split;
+    if (P.bs <= 64) {
+        int n = 0;                                  // splits of sequence `lane` (padding rows get one)
+        if (lane < P.bs) n = max(1, (P.context_lens[lane] + P.chunk - 1) / P.chunk);
+        int before = 0;
+        for (int s = 0; s < P.bs; ++s) {
+            const int ns = __builtin_amdgcn_readlane(n, s);
+            before += s < lane ? ns : 0;
+        }
+        const int j = blockIdx.y;
+        const unsigned long long le = __ballot(lane < P.bs && before <= j);
+        b = __popcll(le) - 1;
+        split = j - __builtin_amdgcn_readlane(before, b);
+        if (split >= __builtin_amdgcn_readlane(n, b)) return;   // past the last pair
+    } else {
+        b = blockIdx.y / P.nsplit;
+        split = blockIdx.y % P.nsplit;
+    }
+
     const int ctx = P.context_lens[b];
     const int n_valid_splits = (ctx + P.chunk - 1) / P.chunk;
-
     if (ctx <= 0) {
-        // graph-padding row: defined output (zeros), written by split 0
+        // graph-padding row: defined output (zeros), written by its split 0
         if (split == 0) {
             for (int e = tid; e < P.sq * HPW * (kHeadDim / 8); e += kThreads) {
                 const int d8 = e % (kHeadDim / 8), h = (e / (kHeadDim / 8)) % HPW, s = e / (kHeadDim / 8) / HPW;
@@ -88,63 +110,94 @@ __global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedP
     st.init();
 
     const int32_t* bt = P.block_table + (int64_t)b * P.bt_stride;
-    const int chunk = tid & 15, trow = tid >> 4;    // 512 threads: one pass stages 32 rows
+    const int chunk = tid & 15, trow = tid >> 4;    // 256 threads: one pass stages 16 rows
     const int n_tiles = (key_end - key_begin + kTileKeys - 1) / kTileKeys;
-    TileRegs<kTileKeys, kThreads> regs;
-    // Pass p of a tile holds keys key0 + 32p .. +31: 32 consecutive keys never straddle a page
-    // (page_size % 32 == 0, key_begin % 32 == 0), so each pass looks its page up once.
-    auto fetch = [&](int t) {
+    // 16 consecutive keys starting at a multiple of 16 never straddle a page (page_size % 32 == 0):
+    // each pass looks its page up once.  The loads are unconditional (rows past the context or on
+    // an invalid page id read row `trow` of page 0 instead and are zeroed when they reach LDS), so
+    // the number of loads in flight is known exactly and waiting for one register set does not
+    // drain the other.
+    struct Staged {
+        TileRegs<kTileKeys, kThreads> regs;
+        unsigned row_ok;       // bit p: this thread's row of pass p holds a real key
+        unsigned pass_ok;      // bit p (uniform): pass p lies on a valid page inside the context
+    };
+    const int64_t safe_off = (int64_t)trow * P.c_st + (int64_t)kvh * P.c_sh + chunk * 8;
+    auto fetch = [&](Staged& sg, int t) {
         const int key0 = key_begin + t * kTileKeys;
+        sg.row_ok = 0;
+        sg.pass_ok = 0;
 #pragma unroll
-        for (int p = 0; p < KW; ++p) {
-            const int kp = key0 + 32 * p;
-            bool ok = kp < key_end;
-            int64_t page = -1;
-            if (ok) {
-                const int page_slot = kp / P.page_size;
-                page = page_slot < P.max_pages ? (int64_t)bt[page_slot] : -1;
-                ok = page >= 0 && page < P.num_pages;
-            }
-            if (ok && kp + trow < key_end) {
-                const int64_t off = page * P.c_sp + (int64_t)(kp % P.page_size + trow) * P.c_st + (int64_t)kvh * P.c_sh + chunk * 8;
-                regs.k[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.k_cache + off));
-                regs.v[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.v_cache + off));
-            } else {                                // past the context or an invalid page id: zero rows
-                regs.k[p] = u32x4{0, 0, 0, 0};
-                regs.v[p] = u32x4{0, 0, 0, 0};
-            }
+        for (int p = 0; p < kPasses; ++p) {
+            const int kp = key0 + 16 * p;
+            const int page_slot = P.page_shift >= 0 ? kp >> P.page_shift : kp / P.page_size;
+            const int in_page = P.page_shift >= 0 ? kp & (P.page_size - 1) : kp % P.page_size;
+            const bool inside = kp < key_end && page_slot < P.max_pages;
+            const int64_t page = bt[inside ? page_slot : 0];
+            const bool ok = inside && page >= 0 && page < P.num_pages;             // uniform
+            const int64_t off = ok ? page * P.c_sp + (int64_t)in_page * P.c_st + safe_off : safe_off;
+            sg.regs.k[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.k_cache + off));
+            sg.regs.v[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.v_cache + off));
+            sg.pass_ok |= (ok ? 1u : 0u) << p;
+            sg.row_ok |= ((ok && kp + trow < key_end) ? 1u : 0u) << p;
         }
     };
-    // Keys of an invalid page are excluded (not merely zeroed): the owning wavefront skips them.
-    auto slice_ok = [&](int kp) {
-        if (kp >= key_end) return false;
-        const int page_slot = kp / P.page_size;
-        const int64_t page = page_slot < P.max_pages ? (int64_t)bt[page_slot] : -1;
-        return page >= 0 && page < P.num_pages;
+    unsigned tile_pass_ok[2] = {0, 0};                 // pass_ok of the tile sitting in LDS buffer 0 / 1
+    auto stage = [&](int buf, Staged& sg) {
+#pragma unroll
+        for (int p = 0; p < kPasses; ++p)
+            if (!((sg.row_ok >> p) & 1u)) { sg.regs.k[p] = u32x4{0, 0, 0, 0}; sg.regs.v[p] = u32x4{0, 0, 0, 0}; }
+        store_tile<kTileKeys, kThreads>(lds[buf], lds[buf] + kTileBytes, sg.regs, tid);
+        tile_pass_ok[buf] = sg.pass_ok;
     };
-
-    fetch(0);
-    for (int t = 0; t < n_tiles; ++t) {
-        __syncthreads();
-        store_tile<kTileKeys, kThreads>(lds_k, lds_v, regs, tid);
-        __syncthreads();
-        if (t + 1 < n_tiles) fetch(t + 1);
-
-        const int key0 = key_begin + t * kTileKeys + kw * 32;        // this wavefront's 32 keys
-        if (slice_ok(key0)) {
+    auto compute = [&](int t) {
+        const char* lk = lds[t & 1];
+        const int key0 = key_begin + t * kTileKeys + kw * 32;        // this wavefront's 32 keys = passes 2kw, 2kw+1
+        // keys of an invalid page are excluded (not merely zeroed): the owning wavefront skips them
+        if ((tile_pass_ok[t & 1] >> (2 * kw)) & 1u) {
             if (key0 + 32 <= key_end)
-                attn_step<1, false>(lds_k, lds_v, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
             else
-                attn_step<1, true>(lds_k, lds_v, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<1, true>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
         }
+    };
+
+    // Register sets ra / rb hold the tiles after the one in LDS; tile t+1 sits in set (t+1)%2.
+    Staged ra, rb;
+    fetch(ra, 0);
+    if (DEPTH == 2 && n_tiles > 1) fetch(rb, 1);
+    stage(0, ra);
+    if (DEPTH == 2) { if (n_tiles > 2) fetch(ra, 2); } else { if (n_tiles > 1) fetch(ra, 1); }
+    __syncthreads();
+    for (int t = 0; t < n_tiles; t += 2) {
+        // even tile t from buffer 0; stage tile t+1 into buffer 1
+        compute(t);
+        if (t + 1 < n_tiles) {
+            if (DEPTH == 2) {
+                stage(1, rb);
+                if (t + 3 < n_tiles) fetch(rb, t + 3);
+            } else {
+                stage(1, ra);
+                if (t + 2 < n_tiles) fetch(ra, t + 2);
+            }
+        }
+        __syncthreads();
+        if (t + 1 >= n_tiles) break;
+        // odd tile t+1 from buffer 1; stage tile t+2 into buffer 0
+        compute(t + 1);
+        if (t + 2 < n_tiles) {
+            stage(0, ra);
+            if (DEPTH == 2) { if (t + 4 < n_tiles) fetch(ra, t + 4); } else { if (t + 3 < n_tiles) fetch(ra, t + 3); }
+        }
+        __syncthreads();
     }
 
     // ---- merge the KW key-slice states of each head (tree through LDS) ----------------------
     st.l = both_halves_sum(st.l);          // a state is now (m, l, O) per query
     // Exchange layout per sending wavefront: O as [4][16][64 lanes] floats, then m, l as [64].
     constexpr int kStateFloats = 4 * 16 * 64 + 2 * 64;
-    static_assert(4 * kStateFloats * 4 <= (int)sizeof(lds), "merge buffer exceeds the tile region");
-    float* xch = reinterpret_cast<float*>(lds);
+    static_assert(HPW * (KW / 2) * kStateFloats * 4 <= (int)sizeof(lds), "merge buffer exceeds the tile region");
+    float* xch = reinterpret_cast<float*>(&lds[0][0]);
     auto send = [&](int slot) {
         float* dst = xch + slot * kStateFloats;
 #pragma unroll
@@ -168,14 +221,13 @@ __global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedP
             for (int i = 0; i < 16; ++i)
                 st.o[t][i] = st.o[t][i] * a1 + src[(t * 16 + i) * 64 + lane] * a2;
     };
-    __syncthreads();                         // tiles no longer needed
+    // (the loop's last barrier already separates the tile reads from these writes)
 #pragma unroll
     for (int stride = KW / 2; stride >= 1; stride >>= 1) {
-        const int slot = (wave / KW) * stride + (kw - stride);     // 4 slots at most (HPW * KW/2)
-        if (kw >= stride && kw < 2 * stride) send(slot);
+        if (kw >= stride && kw < 2 * stride) send((wave / KW) * stride + (kw - stride));
         __syncthreads();
         if (kw < stride) recv((wave / KW) * stride + kw);
-        __syncthreads();
+        if (stride > 1) __syncthreads();
     }
     if (kw != 0 || !row_ok) return;
 
@@ -211,11 +263,11 @@ __global__ __launch_bounds__(kThreads) void paged_block_attn_kernel(const PagedP
 }
 
 // One wavefront per (sequence, head, query): merges the split partials.
-__global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P, int bs)
+__global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t n_rows = (int64_t)bs * P.num_q_heads * P.sq;
+    const int64_t n_rows = (int64_t)P.bs * P.num_q_heads * P.sq;
     if (row >= n_rows) return;
     const int s = (int)(row % P.sq);
     const int hq = (int)((row / P.sq) % P.num_q_heads);
@@ -299,7 +351,6 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     if (bs == 0 || sq == 0) return MDX_OK;
     MDX_REQUIRE(max_pages > 0, MDX_EINVAL, "paged_block_attn: empty block table");
     MDX_REQUIRE(q && o && k_cache && v_cache && block_table && context_lens, MDX_EINVAL, "paged_block_attn: null pointer");
-    MDX_REQUIRE(bs <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: bs %d > 65535", bs);
     MDX_REQUIRE(bt_stride >= max_pages, MDX_EINVAL, "paged_block_attn: bt_stride < max_pages");
     MDX_REQUIRE(mdx::aligned16(q) && mdx::aligned16(o) && mdx::aligned16(k_cache) && mdx::aligned16(v_cache) &&
                 q_stride_b % 8 == 0 && q_stride_s % 8 == 0 && q_stride_h % 8 == 0 &&
@@ -315,7 +366,9 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     P.o_sb = o_stride_b; P.o_ss = o_stride_s; P.o_sh = o_stride_h;
     P.c_sp = cache_stride_page; P.c_st = cache_stride_tok; P.c_sh = cache_stride_head;
     P.block_table = block_table; P.bt_stride = bt_stride; P.context_lens = context_lens;
-    P.sq = sq; P.heads_per_kv = G; P.page_size = page_size; P.max_pages = max_pages; P.num_pages = num_pages;
+    P.bs = bs; P.sq = sq; P.heads_per_kv = G; P.page_size = page_size; P.max_pages = max_pages;
+    P.page_shift = -1;
+    for (int i = 0; i < 31; ++i) if (page_size == (1 << i)) P.page_shift = i; P.num_pages = num_pages;
     P.chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size);
     P.nsplit = nsplit_of(max_pages, page_size, P.chunk);
     P.num_q_heads = num_q_heads;
@@ -330,12 +383,14 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
         P.part_o = static_cast<float*>(workspace);
         P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
     }
-    const dim3 grid((unsigned)P.nsplit, (unsigned)(num_q_heads / HPW), (unsigned)bs);
-    if (HPW == 2) paged_block_attn_kernel<2><<<grid, kThreads, 0, stream>>>(P);
-    else          paged_block_attn_kernel<1><<<grid, kThreads, 0, stream>>>(P);
+    // head group fastest, then the dense (sequence, split) index
+    MDX_REQUIRE((int64_t)bs * P.nsplit <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: bs * splits %lld > 65535", (long long)bs * P.nsplit);
+    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)(bs * P.nsplit));
+    if (HPW == 2) paged_block_attn_kernel<2, 2><<<grid, kThreads, 0, stream>>>(P);
+    else          paged_block_attn_kernel<1, 1><<<grid, kThreads, 0, stream>>>(P);
     int rc = mdx::check_launch("paged_block_attn");
     if (rc != MDX_OK || P.nsplit == 1) return rc;
     const int64_t n_rows = (int64_t)bs * num_q_heads * sq;
-    paged_combine_kernel<<<(unsigned)((n_rows + 3) / 4), 256, 0, stream>>>(P, bs);
+    paged_combine_kernel<<<(unsigned)((n_rows + 3) / 4), 256, 0, stream>>>(P);
     return mdx::check_launch("paged_combine");
 }
