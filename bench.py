@@ -45,21 +45,34 @@ def ev_pair():
 
 
 def time_kernel(fn, warmup, iters):
-    """Average duration (ms) of fn's GPU work, HIP events on the launch stream (torch's current
-    stream, which is where libmdx enqueues), one event pair per call."""
+    """Average duration (ms) of fn's GPU work.  fn(i) must only enqueue work (no allocation, no
+    host sync); the `iters` calls are bracketed by ONE pair of HIP events recorded on the launch
+    stream (torch's current stream, which is where libmdx enqueues), so the quotient is the
+    back-to-back launch duration with the host running ahead of the GPU.  A second number,
+    the minimum over individually bracketed launches, is returned for reference."""
     for _ in range(warmup):
         fn(0)
     torch.cuda.synchronize()
-    pairs = []
+    a, b = ev_pair()
+    a.record()
     for i in range(iters):
-        a, b = ev_pair()
-        a.record()
         fn(i)
-        b.record()
-        pairs.append((a, b))
+    b.record()
     torch.cuda.synchronize()
-    ts = [a.elapsed_time(b) for a, b in pairs]
-    return float(np.mean(ts)), float(np.min(ts))
+    avg = a.elapsed_time(b) / iters
+    pairs = []
+    for i in range(min(iters, 10)):
+        x, y = ev_pair()
+        x.record()
+        fn(i)
+        y.record()
+        pairs.append((x, y))
+    torch.cuda.synchronize()
+    return float(avg), float(min(x.elapsed_time(y) for x, y in pairs))
+
+
+def raw_stream():
+    return torch.cuda.current_stream().cuda_stream
 
 
 # ----------------------------------------------------------------------------- config 3
@@ -237,11 +250,15 @@ def main():
     attn.k_cache, attn.v_cache = g3["k_cache"], g3["v_cache"]
     mdx.set_context(True, g3["cu"], g3["cu"], max_len, max_len, g3["slots"], None, None, block_size=S)
 
-    def attn_only(_):
-        return mdx.sparse_attn_varlen(g3["q"], g3["k"], g3["v"], g3["cu"], g3["cu"], S, max_seqlen=max_len)
+    o3 = torch.empty_like(g3["q"])
 
-    def store_only(_):
-        mdx.store_kvcache(g3["k"], g3["v"], g3["k_cache"], g3["v_cache"], g3["slots"])
+    def attn_only(_):
+        q, k, v = g3["q"], g3["k"], g3["v"]
+        rc = mdx.lib().mdx_staircase_attn_varlen(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
+            v.stride(0), v.stride(1), o3.stride(0), o3.stride(1), g3["cu"].data_ptr(), g3["cu"].data_ptr(), len(host3["lens"]),
+            max_len, q.shape[0], HQ, HKV, D, S, 1 / math.sqrt(D), 0, raw_stream())
+        assert rc == 0
 
     ms_step = attn_ms = float("nan")
     if want("step"):
@@ -260,12 +277,30 @@ def main():
             roofline=dict(bound="mfma", achieved=round(work3["flops"] / attn_ms / 1e9, 2), peak=PEAK_MFMA_TFLOPS,
                           unit="TFLOP/s", frac=round(work3["flops"] / attn_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), traffic=None))
     if want("store"):
+        # three rotating (source, cache) sets, about 900 MB touched per round trip, so the 256 MB
+        # last-level cache cannot serve the next launch; the C ABI is called directly
+        L = mdx.lib()
+        N = g3["k"].shape[0]
+        sets = [(g3["k"], g3["v"], g3["k_cache"], g3["v_cache"])]
+        for _ in range(2):
+            f2 = host3["fused"].to(dev)
+            sets.append((f2[:, HQ * D:(HQ + HKV) * D].reshape(N, HKV, D).contiguous(), f2[:, (HQ + HKV) * D:].view(N, HKV, D),
+                         torch.zeros_like(g3["k_cache"]), torch.zeros_like(g3["v_cache"])))
+        num_slots = g3["k_cache"].shape[0] * PAGE
+        stream = raw_stream()
+
+        def store_only(i):
+            k, v, kc, vc = sets[i % 3]
+            L.mdx_store_kvcache(k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0), kc.data_ptr(), vc.data_ptr(),
+                                g3["slots"].data_ptr(), N, HKV * D, 2, num_slots, stream)
         st_ms, st_min = time_kernel(store_only, W, K)
         gbs = work3["store_bytes"] / st_ms / 1e6
         result_ops["store_kvcache"] = dict(
             ms=round(st_ms, 4), ms_min=round(st_min, 4),
             roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                           frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        del sets
+        torch.cuda.empty_cache()
     mdx.reset_context()
 
     # ---------------- config 2: paged single-block attention ---------------------------------------
@@ -273,10 +308,21 @@ def main():
         log("[bench] building config 2 inputs (64 GiB page pool, referenced pages only are filled)")
         c2 = make_cfg2(dev)
 
+        L = mdx.lib()
+        bs2, maxp = c2["tables"][0].shape
+        ws_bytes = L.mdx_paged_block_attn_workspace_bytes(bs2, S, HQ, HKV, D, maxp, PAGE)
+        ws2 = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        o2 = torch.empty_like(c2["q"])
+        kc2, vc2, q2 = c2["k_cache"], c2["v_cache"], c2["q"]
+
         def paged(i):
-            return mdx.flash_attn_with_kvcache(c2["q"], c2["k_cache"], c2["v_cache"], cache_seqlens=c2["lens"],
-                                               block_table=c2["tables"][i % len(c2["tables"])],
-                                               softmax_scale=1 / math.sqrt(D), causal=False)
+            bt = c2["tables"][i % len(c2["tables"])]
+            rc = L.mdx_paged_block_attn(q2.data_ptr(), o2.data_ptr(), kc2.data_ptr(), vc2.data_ptr(),
+                                        q2.stride(0), q2.stride(1), q2.stride(2), o2.stride(0), o2.stride(1), o2.stride(2),
+                                        kc2.stride(0), kc2.stride(1), kc2.stride(2), bt.data_ptr(), bt.stride(0),
+                                        c2["lens"].data_ptr(), bs2, S, HQ, HKV, D, maxp, PAGE, kc2.shape[0],
+                                        1 / math.sqrt(D), 0, ws2.data_ptr(), ws_bytes, raw_stream())
+            assert rc == 0
         pg_ms, pg_min = time_kernel(paged, W, K)
         gbs = c2["work"]["bytes"] / pg_ms / 1e6
         result_ops["paged_block_attn"] = dict(
@@ -293,20 +339,31 @@ def main():
         log("[bench] building config 4 inputs")
         c4 = make_cfg4(dev)
         cfg4_tokens = c4["tokens"]
-        dtok = [c4["tokens"].clone().to(dev) for _ in range(K + W + 1)]
-        state = {"i": 0}
+        L = mdx.lib()
+        rows4 = 32 * S
+        ws_bytes4 = L.mdx_confidence_argmax_workspace_bytes(rows4, VOCAB)
+        ws4 = torch.empty(max(ws_bytes4, 16), dtype=torch.uint8, device=dev)
+        tok0 = c4["tokens"].to(dev)
+        dtok = tok0.clone()
+        x0_4 = torch.empty(32, S, dtype=torch.int64, device=dev)
+        p_4 = torch.empty(32, S, dtype=torch.float32, device=dev)
+        tr_4 = torch.empty(32, S, dtype=torch.uint8, device=dev)
+        cnt_4 = torch.empty(32, dtype=torch.int32, device=dev)
 
         def unmask(i):
-            t = dtok[state["i"] % len(dtok)]
-            state["i"] += 1
-            return mdx.unmask_step(c4["logits"][i % len(c4["logits"])], t, MASK_ID, 0.9, 4)
+            lg = c4["logits"][i % len(c4["logits"])]
+            dtok.copy_(tok0)                       # every step starts from the same masked block (8 KB copy)
+            rc = L.mdx_unmask_step(lg.data_ptr(), VOCAB, 0, None, None, 0, dtok.data_ptr(), MASK_ID, 0.9, 4,
+                                   x0_4.data_ptr(), p_4.data_ptr(), tr_4.data_ptr(), cnt_4.data_ptr(), 32, S, VOCAB,
+                                   ws4.data_ptr(), ws_bytes4, raw_stream())
+            assert rc == 0
         um_ms, um_min = time_kernel(unmask, W, K)
         gbs = c4["bytes"] / um_ms / 1e6
         result_ops["unmask_step"] = dict(
             ms=round(um_ms, 4), ms_min=round(um_min, 4),
             roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
                           frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
-        del c4, dtok
+        del c4
         torch.cuda.empty_cache()
 
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
