@@ -164,6 +164,39 @@ def make_cfg4(dev, n_sets=2, seed=4):
     return dict(logits=sets, tokens=tokens, bytes=32 * S * VOCAB * 2)
 
 
+# ----------------------------------------------------------------------------- config 5
+def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8):
+    """Random-init SDAR-shaped decoder (28 layers, hidden 2048, Hq 16 / Hkv 8 / d 128, SwiGLU 6144,
+    vocab 151936), batch 32, 1024 random prefix embeddings + 64 prompt tokens per sequence, 2048 new
+    tokens in 32-token blocks, k = 32/8 = 4 committed positions per denoising pass, threshold 0.9.
+    Returns committed tokens/s over the whole generation (prefill included)."""
+    from mdx.engine import BlockDiffusionEngine, Decoder, DecoderConfig, SamplingParams
+    cfg = DecoderConfig(num_layers=layers)
+    model = Decoder(cfg, dev, seed=5)
+    pages_per_seq = (1088 + new_tokens + PAGE - 1) // PAGE + 1
+    eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5)
+    g = torch.Generator().manual_seed(5)
+    sp = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True, transfer_count=S // steps_per_block)
+    for _ in range(batch):
+        ids = [0] * 1024 + torch.randint(0, 151000, (64,), generator=g).tolist()
+        eng.add_request(ids, sp, prefix_embeds=(torch.randn(1024, cfg.hidden_size, generator=g) * 0.02).to(dev))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    seqs = eng.generate()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    done = sum(s.num_completion_tokens for s in seqs)
+    st = eng.stats
+    out = dict(tokens_per_s=round(done / dt, 1), seconds=round(dt, 3), committed_tokens=done, batch=batch,
+               prefill_passes=st["prefill_passes"], decode_passes=st["decode_passes"],
+               prefill_s=round(st["prefill_s"], 3), decode_s=round(st["decode_s"], 3),
+               ms_per_decode_pass=round(st["decode_s"] / max(1, st["decode_passes"]) * 1e3, 3), layers=layers,
+               model="random-init 28-layer SDAR-shaped decoder, stock PyTorch-ROCm GEMMs, libmdx attention/KV store/unmask")
+    del eng, model
+    torch.cuda.empty_cache()
+    return out
+
+
 # ----------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(host3):
     """The oracle on the host cores, bounded: one config-3 sequence of 4096 tokens through SDPA
@@ -225,7 +258,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
-    ap.add_argument("--only", default="", help="comma list of legs to run: step,store,paged,unmask (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: step,store,paged,unmask,decode (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -366,6 +399,14 @@ def main():
         del c4
         torch.cuda.empty_cache()
 
+    # ---------------- config 5: end-to-end block-diffusion decode ---------------------------------------
+    decode = None
+    if want("decode"):
+        log("[bench] config 5: end-to-end block-diffusion decode (32 x 2048 tokens)")
+        del g3, attn
+        torch.cuda.empty_cache()
+        decode = run_cfg5(dev)
+
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
     cpu = None
     if not args.skip_cpu:
@@ -392,6 +433,7 @@ def main():
         "roofline": result_ops.get("staircase_attn", {}).get("roofline"),
         "cpu_baseline": cpu,
         "ops": result_ops,
+        "decode": decode,
         "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
     }
     print(json.dumps(line), flush=True)

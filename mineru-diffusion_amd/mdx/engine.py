@@ -1,0 +1,429 @@
+"""A minimal block-diffusion decode loop around the mdx hot path.
+
+This is the caller side of the hot path, restated from the nano_dvlm engine so that the
+kernels can be driven exactly as the engine drives them:
+
+  Sequence / slot arithmetic      nanovllm/engine/sequence.py:16-141
+  page allocation                 nanovllm/engine/block_manager.py:59-102 (no prefix hashing: it is
+                                  disabled in the reference, block_manager.py:65-66)
+  prepare_prefill / prepare_decode nanovllm/engine/model_runner.py:121-185
+  denoise -> CACHING -> append    nanovllm/engine/scheduler.py:24-82
+  decoder layer structure         nanovllm/models/sdar.py:68-181, layers/layernorm.py:16-40,
+                                  layers/rotary_embedding.py:6-48, layers/embed_head.py:61-67
+
+The decoder is a random-init scaffold built from stock PyTorch ops (its GEMMs are library
+GEMMs); attention, the KV store and the unmask step go through libmdx.  There is no vision
+tower, tokenizer, weight loader or tensor parallelism here.
+"""
+from __future__ import annotations
+
+import math
+import time
+from collections import deque
+from dataclasses import dataclass, field
+from enum import Enum, auto
+from itertools import count
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .context import get_context, reset_context, set_context
+from .layers import Attention
+from .ops import unmask_step
+
+PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
+
+
+# ----------------------------------------------------------------------------- requests
+@dataclass
+class SamplingParams:
+    """nanovllm/sampling_params.py:4-15 plus the number of positions committed per step when
+    fewer exceed the threshold (1 in the engine, block/steps in the HF generate loop)."""
+    temperature: float = 1.0
+    max_new_tokens: int = 64
+    ignore_eos: bool = False
+    denoising_strategy: str = "low_confidence_dynamic"
+    dynamic_threshold: float = 0.9
+    stop_token_ids: list = field(default_factory=list)
+    transfer_count: int = 1
+
+    def __post_init__(self):
+        assert self.temperature > 1e-10, "greedy sampling is not permitted"
+
+
+class SequenceStatus(Enum):
+    WAITING = auto()
+    RUNNING = auto()
+    CACHING = auto()
+    FINISHED = auto()
+
+
+class Sequence:
+    """Per-request state (sequence.py:16-141).  `prefix_embeds` ([n, hidden]) replaces the input
+    embeddings of the first n prompt tokens (the engine splices vision embeddings there)."""
+    counter = count()
+
+    def __init__(self, token_ids, sampling_params=None, denoising_block_size=32, mask_token_id=151669,
+                 prefix_embeds: torch.Tensor | None = None):
+        self.seq_id = next(Sequence.counter)
+        self.status = SequenceStatus.WAITING
+        self.token_ids = list(token_ids)
+        self.step_map = []
+        self.num_tokens = len(self.token_ids)            # committed tokens, no mask tokens
+        self.num_prompt_tokens = len(self.token_ids)
+        self.block_table: list[int] = []
+        self.sampling_params = sampling_params or SamplingParams()
+        self.temperature = self.sampling_params.temperature
+        self.max_new_tokens = self.sampling_params.max_new_tokens
+        self.ignore_eos = self.sampling_params.ignore_eos
+        self.denoising_block_size = denoising_block_size
+        self.mask_token_id = mask_token_id
+        self.prefix_embeds = prefix_embeds
+        self.current_denoising_block = torch.full((denoising_block_size,), mask_token_id, dtype=torch.int64)
+        self.current_step_map = torch.zeros((denoising_block_size,), dtype=torch.int32)
+        self.current_denoise_step = 0
+
+    def __len__(self):
+        return self.num_tokens
+
+    @property
+    def is_finished(self):
+        return self.status == SequenceStatus.FINISHED
+
+    @property
+    def is_caching(self):
+        return self.status == SequenceStatus.CACHING
+
+    @property
+    def num_completion_tokens(self):
+        return self.num_tokens - self.num_prompt_tokens
+
+    @property
+    def completion_token_ids(self):
+        return self.token_ids[self.num_prompt_tokens:]
+
+    @property
+    def num_blocks(self):
+        return (self.num_tokens + PAGE - 1) // PAGE
+
+    def append_block(self):                               # sequence.py:97-101
+        self.token_ids.extend(self.current_denoising_block.tolist())
+        self.step_map.extend(self.current_step_map.tolist())
+        self.num_tokens += self.denoising_block_size
+        self.current_denoising_block = torch.full((self.denoising_block_size,), self.mask_token_id, dtype=torch.int64)
+
+    def need_new_block(self):                             # sequence.py:114-115
+        return self.num_tokens + self.denoising_block_size > PAGE * len(self.block_table)
+
+    def get_slots(self, lo: int, hi: int):                # sequence.py:117-141
+        if not self.block_table:
+            return [-1] * (hi - lo)
+        t = torch.arange(lo, hi)
+        table = torch.tensor(self.block_table, dtype=torch.int64)
+        return (table[t // PAGE] * PAGE + t % PAGE).tolist()
+
+
+class BlockManager:
+    """Free-list page allocator (block_manager.py:59-102 without the disabled prefix cache)."""
+
+    def __init__(self, num_pages: int, shuffle_seed: int | None = None):
+        ids = list(range(num_pages))
+        if shuffle_seed is not None:                      # exercise non-contiguous page tables
+            g = torch.Generator().manual_seed(shuffle_seed)
+            ids = torch.randperm(num_pages, generator=g).tolist()
+        self.free = deque(ids)
+
+    def can_allocate(self, seq):
+        return len(self.free) >= seq.num_blocks
+
+    def allocate(self, seq):
+        assert not seq.block_table
+        seq.block_table.extend(self.free.popleft() for _ in range(seq.num_blocks))
+
+    def can_append(self, seq):
+        return len(self.free) >= int(seq.need_new_block())
+
+    def may_append(self, seq):
+        if seq.need_new_block():
+            seq.block_table.append(self.free.popleft())
+
+    def deallocate(self, seq):
+        self.free.extend(reversed(seq.block_table))
+        seq.block_table.clear()
+
+
+# ----------------------------------------------------------------------------- decoder scaffold
+@dataclass
+class DecoderConfig:
+    """Defaults = the language model of mineru_diffusion/configuration_mineru_diffusion.py:12-27."""
+    num_layers: int = 28
+    hidden_size: int = 2048
+    num_heads: int = 16
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    intermediate_size: int = 6144
+    vocab_size: int = 151936
+    rope_theta: float = 1.0e6
+    rms_norm_eps: float = 1e-6
+    max_position: int = 8192
+    block_size: int = 32
+    mask_token_id: int = 151669
+
+
+def _rms(x, w, eps):
+    return F.rms_norm(x, (x.shape[-1],), w, eps)
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, c: DecoderConfig):
+        super().__init__()
+        self.c = c
+        qkv_out = (c.num_heads + 2 * c.num_kv_heads) * c.head_dim
+        self.qkv_proj = nn.Parameter(torch.empty(qkv_out, c.hidden_size))
+        self.o_proj = nn.Parameter(torch.empty(c.hidden_size, c.num_heads * c.head_dim))
+        self.gate_up_proj = nn.Parameter(torch.empty(2 * c.intermediate_size, c.hidden_size))
+        self.down_proj = nn.Parameter(torch.empty(c.hidden_size, c.intermediate_size))
+        self.q_norm = nn.Parameter(torch.ones(c.head_dim))
+        self.k_norm = nn.Parameter(torch.ones(c.head_dim))
+        self.input_layernorm = nn.Parameter(torch.ones(c.hidden_size))
+        self.post_attention_layernorm = nn.Parameter(torch.ones(c.hidden_size))
+        self.attn = Attention(c.num_heads, c.head_dim, c.head_dim ** -0.5, c.num_kv_heads)
+
+    def forward(self, positions, x, residual, cos, sin):
+        c = self.c
+        if residual is None:                               # sdar.py:147-150
+            residual = x
+            h = _rms(x, self.input_layernorm, c.rms_norm_eps)
+        else:
+            residual = x + residual
+            h = _rms(residual, self.input_layernorm, c.rms_norm_eps)
+        qkv = F.linear(h, self.qkv_proj)
+        q_size, kv_size = c.num_heads * c.head_dim, c.num_kv_heads * c.head_dim
+        q, k, v = qkv.split([q_size, kv_size, kv_size], dim=-1)
+        shape = (*positions.shape, -1, c.head_dim)
+        q, k, v = q.view(shape), k.view(shape), v.view(shape)   # v stays a strided view of qkv
+        q = _rms(q, self.q_norm, c.rms_norm_eps)
+        k = _rms(k, self.k_norm, c.rms_norm_eps)
+        q, k = _rope(q, cos, sin), _rope(k, cos, sin)
+        o = self.attn(q, k, v)
+        x = F.linear(o, self.o_proj)
+        residual = x + residual
+        h = _rms(residual, self.post_attention_layernorm, c.rms_norm_eps)
+        gate, up = F.linear(h, self.gate_up_proj).chunk(2, dim=-1)
+        return F.linear(F.silu(gate) * up, self.down_proj), residual
+
+
+def _rope(x, cos, sin):                                    # rotary_embedding.py:6-14
+    x1, x2 = torch.chunk(x.float(), 2, dim=-1)
+    return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1).to(x.dtype)
+
+
+class Decoder(nn.Module):
+    """SDAR-shaped decoder-only model (sdar.py:157-216) with random weights (std 0.02)."""
+
+    def __init__(self, c: DecoderConfig, device, dtype=torch.bfloat16, seed: int = 0):
+        super().__init__()
+        self.c = c
+        self.embed_tokens = nn.Parameter(torch.empty(c.vocab_size, c.hidden_size))
+        self.layers = nn.ModuleList(DecoderLayer(c) for _ in range(c.num_layers))
+        self.norm = nn.Parameter(torch.ones(c.hidden_size))
+        self.lm_head = nn.Parameter(torch.empty(c.vocab_size, c.hidden_size))
+        self.to(device=device, dtype=dtype)
+        g = torch.Generator(device=device).manual_seed(seed)
+        with torch.no_grad():
+            for name, p in self.named_parameters():
+                if p.dim() == 2:
+                    p.normal_(0.0, 0.02, generator=g)
+        inv_freq = 1.0 / (c.rope_theta ** (torch.arange(0, c.head_dim, 2, dtype=torch.float) / c.head_dim))
+        freqs = torch.einsum("i,j->ij", torch.arange(c.max_position, dtype=torch.float), inv_freq)
+        self.register_buffer("cos", freqs.cos().to(device), persistent=False)
+        self.register_buffer("sin", freqs.sin().to(device), persistent=False)
+
+    def embed(self, input_ids):
+        return F.embedding(input_ids, self.embed_tokens)
+
+    @torch.inference_mode()
+    def forward(self, inputs_embeds, positions):
+        cos = self.cos[positions].unsqueeze(-2)
+        sin = self.sin[positions].unsqueeze(-2)
+        x, residual = inputs_embeds, None
+        for layer in self.layers:
+            x, residual = layer(positions, x, residual, cos, sin)
+        return _rms(x + residual, self.norm, self.c.rms_norm_eps)
+
+    @torch.inference_mode()
+    def compute_logits(self, hidden):                      # embed_head.py:61-67
+        ctx = get_context()
+        if ctx.is_prefill:
+            starts = ctx.cu_seqlens_q[1:] - self.c.block_size
+            idx = starts.unsqueeze(1) + torch.arange(self.c.block_size, device=starts.device)
+            hidden = hidden[idx.long()].contiguous()
+        return F.linear(hidden, self.lm_head)
+
+
+# ----------------------------------------------------------------------------- engine
+class BlockDiffusionEngine:
+    """Scheduler + runner for block-diffusion decoding (llm_engine.py:66-73 `step`, scheduler.py,
+    model_runner.py:127-219), one GPU, eager."""
+
+    def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
+                 max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None):
+        self.model = model
+        self.c = model.c
+        self.device = model.lm_head.device
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_num_seqs = max_num_seqs
+        self.block_manager = BlockManager(num_pages, shuffle_pages_seed)
+        self.waiting: deque[Sequence] = deque()
+        self.running: deque[Sequence] = deque()
+        self.on_logits = on_logits                         # test hook: (is_prefill, seqs, logits)
+        self.unmask = unmask or unmask_step                # the device unmask step (replaceable in host-only tests)
+        c = self.c
+        dtype = model.lm_head.dtype
+        # KV pool [2, layers, pages, 256, Hkv, d] (model_runner.py:113-119)
+        self.kv_cache = torch.zeros(2, max(c.num_layers, 1), num_pages, PAGE, c.num_kv_heads, c.head_dim, dtype=dtype, device=self.device)
+        for i, layer in enumerate(model.layers):
+            layer.attn.k_cache = self.kv_cache[0, i]
+            layer.attn.v_cache = self.kv_cache[1, i]
+        self.stats = dict(prefill_passes=0, decode_passes=0, committed_tokens=0, prefill_s=0.0, decode_s=0.0)
+
+    # ---- requests / scheduling (scheduler.py:21-63) ----
+    def add_request(self, token_ids, sampling_params=None, prefix_embeds=None) -> Sequence:
+        seq = Sequence(token_ids, sampling_params, self.c.block_size, self.c.mask_token_id, prefix_embeds)
+        self.waiting.append(seq)
+        return seq
+
+    def is_finished(self):
+        return not self.waiting and not self.running
+
+    def schedule(self):
+        scheduled, tokens = [], 0
+        while self.waiting and len(scheduled) < self.max_num_seqs:
+            seq = self.waiting[0]
+            if tokens + len(seq) > self.max_num_batched_tokens or not self.block_manager.can_allocate(seq):
+                break
+            self.block_manager.allocate(seq)
+            tokens += len(seq)
+            seq.status = SequenceStatus.RUNNING
+            self.waiting.popleft()
+            self.running.append(seq)
+            scheduled.append(seq)
+        if scheduled:
+            return scheduled, True
+        for seq in list(self.running)[: self.max_num_seqs]:
+            if not self.block_manager.can_append(seq):
+                raise RuntimeError("KV pool exhausted (preemption is not part of this scaffold)")
+            self.block_manager.may_append(seq)
+            scheduled.append(seq)
+        assert scheduled
+        return scheduled, False
+
+    def postprocess(self, seqs):                           # scheduler.py:65-82
+        for seq in seqs:
+            if not seq.is_caching:
+                if not (seq.current_denoising_block == seq.mask_token_id).any():
+                    seq.status = SequenceStatus.CACHING
+                continue
+            finished = any((seq.current_denoising_block == s).any() for s in seq.sampling_params.stop_token_ids)
+            seq.append_block()
+            self.stats["committed_tokens"] += seq.denoising_block_size
+            if (not seq.ignore_eos and finished) or seq.num_completion_tokens >= seq.max_new_tokens:
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)
+            else:
+                seq.status = SequenceStatus.RUNNING
+
+    # ---- runner (model_runner.py:121-219) ----
+    def _block_tables(self, seqs):
+        n = max(len(s.block_table) for s in seqs)
+        bt = torch.full((len(seqs), n), -1, dtype=torch.int32)
+        for i, s in enumerate(seqs):
+            bt[i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
+        return bt.to(self.device, non_blocking=True)
+
+    def _embed(self, seqs, input_ids, is_prefill):
+        emb = self.model.embed(input_ids)
+        if is_prefill:
+            at = 0
+            for s in seqs:
+                if s.prefix_embeds is not None:
+                    n = s.prefix_embeds.shape[0]
+                    emb[at:at + n] = s.prefix_embeds.to(emb.dtype)
+                at += len(s) + self.c.block_size
+        return emb
+
+    def prepare_prefill(self, seqs):                       # model_runner.py:127-167 (no prefix cache)
+        S = self.c.block_size
+        ids, pos, slots, cu, max_len = [], [], [], [0], 0
+        for s in seqs:
+            n = len(s) + S
+            ids.extend(s.token_ids + s.current_denoising_block.tolist())
+            pos.extend(range(n))
+            cu.append(cu[-1] + n)
+            max_len = max(max_len, n)
+            slots.extend(s.get_slots(0, len(s)) + [-1] * S)
+        dev = self.device
+        cu = torch.tensor(cu, dtype=torch.int32).to(dev, non_blocking=True)
+        set_context(True, cu, cu, max_len, max_len, torch.tensor(slots, dtype=torch.int32).to(dev, non_blocking=True),
+                    None, None, block_size=S)
+        return (torch.tensor(ids, dtype=torch.int64).to(dev, non_blocking=True),
+                torch.tensor(pos, dtype=torch.int64).to(dev, non_blocking=True))
+
+    def prepare_decode(self, seqs):                        # model_runner.py:169-185
+        S = self.c.block_size
+        ids = torch.stack([s.current_denoising_block for s in seqs])
+        lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
+        pos = lens.unsqueeze(1) + torch.arange(S)
+        slots = torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32)
+        dev = self.device
+        set_context(False, slot_mapping=slots.to(dev, non_blocking=True),
+                    context_lens=(lens + S).to(torch.int32).to(dev, non_blocking=True),
+                    block_tables=self._block_tables(seqs), block_size=S)
+        return ids.to(dev, non_blocking=True), pos.to(dev, non_blocking=True)
+
+    def sample(self, logits, seqs) -> int:                 # layers/sampler.py:24-61 on the device
+        sp = seqs[0].sampling_params
+        if sp.denoising_strategy != "low_confidence_dynamic":
+            raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
+        x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
+        temps = torch.tensor([s.temperature for s in seqs], dtype=torch.float32, device=self.device)
+        _, _, transfer, count = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
+                                            temperatures=temps)
+        x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
+        for i, s in enumerate(seqs):
+            s.current_denoising_block = x_cpu[i]
+            s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
+            s.current_denoise_step += 1
+        return int(count.sum().item())
+
+    @torch.inference_mode()
+    def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
+        ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+        hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
+        logits = self.model.compute_logits(hidden)
+        if is_prefill:
+            logits = logits.view(len(seqs), self.c.block_size, -1)
+        if self.on_logits is not None:
+            self.on_logits(is_prefill, seqs, logits)
+        n = self.sample(logits, seqs)
+        reset_context()
+        return n
+
+    def step(self):                                        # llm_engine.py:66-73
+        seqs, is_prefill = self.schedule()
+        t0 = time.perf_counter()
+        n = self.run(seqs, is_prefill)
+        self.postprocess(seqs)
+        dt = time.perf_counter() - t0
+        self.stats["prefill_passes" if is_prefill else "decode_passes"] += 1
+        self.stats["prefill_s" if is_prefill else "decode_s"] += dt
+        return n, is_prefill
+
+    def generate(self):
+        """Runs every queued request to completion; returns them in arrival order."""
+        seqs = list(self.waiting)
+        while not self.is_finished():
+            self.step()
+        return seqs

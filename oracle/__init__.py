@@ -29,6 +29,8 @@ confidence_argmax           torch.softmax / torch.argmax, fp64 explicit sums
 select_transfer             torch.topk on tie-free inputs, brute force over all
                             subsets on 6 positions, counting invariants
 slot_of / get_slots         brute force token-by-token formula
+dense_forward               built from the pinned attention oracle and plain matmuls; its mask
+                            and SDPA are the functions above
 ==========================  =====================================================
 
 The third-party arithmetic behind the reference's paged decode call
@@ -44,3 +46,4 @@ from .staircase import (  # noqa: F401
 from .kvstore import store_kvcache  # noqa: F401
 from .unmask import confidence_argmax, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
 from .slots import slot_of, get_slots  # noqa: F401
+from .engine import dense_forward, expected_passes  # noqa: F401

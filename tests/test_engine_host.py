@@ -1,0 +1,132 @@
+"""Host logic of the mini engine on the CPU: slot arithmetic, page allocation, the tensors the
+runner hands to the kernels, and the denoise -> CACHING -> append state machine, driven by a
+scripted model and an oracle-backed unmask step (no GPU, no libmdx call)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from mdx import get_context
+from mdx.engine import PAGE, BlockDiffusionEngine, BlockManager, DecoderConfig, SamplingParams, Sequence, SequenceStatus
+
+MASK = 99
+
+
+def test_get_slots_matches_brute_force():
+    s = Sequence(list(range(700)), mask_token_id=MASK)
+    assert s.get_slots(0, 5) == [-1] * 5                     # no pages yet (warm-up sequences)
+    s.block_table = [7, 2, 9]
+    for lo, hi in [(0, 700), (250, 262), (255, 257), (512, 700), (300, 301), (10, 10)]:
+        assert s.get_slots(lo, hi) == oracle.get_slots(s.block_table, lo, hi)
+
+
+def test_block_manager_and_need_new_block():
+    bm = BlockManager(8)
+    s = Sequence(list(range(500)), mask_token_id=MASK)       # 2 pages for the prompt
+    assert bm.can_allocate(s)
+    bm.allocate(s)
+    assert s.block_table == [0, 1] and len(bm.free) == 6
+    assert s.need_new_block()                                # 500 + 32 > 512
+    bm.may_append(s)
+    assert s.block_table == [0, 1, 2] and not s.need_new_block()
+    bm.deallocate(s)
+    assert len(bm.free) == 8 and not s.block_table
+
+
+class ScriptedModel:
+    """Stands in for the decoder: records the runner's inputs and returns logits whose argmax at
+    block position p is token 10 + p, with a confidence chosen by the test."""
+
+    def __init__(self, vocab=64, peak=0.0):
+        self.c = DecoderConfig(num_layers=0, hidden_size=8, vocab_size=vocab, block_size=32, mask_token_id=MASK)
+        self.lm_head = torch.zeros(1)
+        self.layers = []
+        self.peak = peak
+        self.calls = []
+
+    def embed(self, ids):
+        return torch.zeros(*ids.shape, 8)
+
+    def __call__(self, embeds, positions):
+        ctx = get_context()
+        self.calls.append(dict(prefill=ctx.is_prefill, positions=positions.clone(), slots=ctx.slot_mapping.clone(),
+                               cu=None if ctx.cu_seqlens_q is None else ctx.cu_seqlens_q.clone(),
+                               ctx_lens=None if ctx.context_lens is None else ctx.context_lens.clone(),
+                               tables=None if ctx.block_tables is None else ctx.block_tables.clone()))
+        return embeds
+
+    def compute_logits(self, hidden):
+        n = len(self.calls[-1]["cu"]) - 1 if self.calls[-1]["prefill"] else hidden.shape[0]
+        logits = torch.zeros(n, 32, self.c.vocab_size)
+        for p in range(32):
+            logits[:, p, 10 + p] = 1.0 + 0.01 * p + self.peak      # later positions slightly more confident
+        return logits.view(-1, self.c.vocab_size) if self.calls[-1]["prefill"] else logits
+
+
+def oracle_unmask(logits, x, mask_id, thr, k, temperatures=None):
+    x0, p, tr, new = oracle.unmask_step(logits.double().numpy(), x.numpy(), mask_id, thr, k,
+                                        None if temperatures is None else temperatures.numpy())
+    x.copy_(torch.from_numpy(new))
+    return torch.from_numpy(x0), torch.from_numpy(p), torch.from_numpy(tr), torch.from_numpy(tr.sum(-1).astype(np.int32))
+
+
+def _engine(model, **kw):
+    return BlockDiffusionEngine(model, num_pages=16, unmask=oracle_unmask, **kw)
+
+
+@pytest.mark.parametrize("k", [1, 4])
+def test_topk_schedule_and_state_machine(k):
+    model = ScriptedModel()
+    eng = _engine(model)
+    sp = SamplingParams(max_new_tokens=64, ignore_eos=True, transfer_count=k)
+    s1 = eng.add_request(list(range(300)), sp)
+    s2 = eng.add_request(list(range(40)), sp)
+    eng.generate()
+    # flat logits: top-k branch, so each block needs 32/k denoising passes + 1 caching pass
+    assert len(model.calls) == oracle.expected_passes(32, k, 2)
+    assert model.calls[0]["prefill"] and not any(c["prefill"] for c in model.calls[1:])
+    for s in (s1, s2):
+        assert s.status == SequenceStatus.FINISHED and s.num_completion_tokens == 64
+        assert s.completion_token_ids == [10 + p for p in range(32)] * 2
+        # most confident positions (the last ones) are committed first
+        assert s.step_map[31] < s.step_map[0]
+    assert len(eng.block_manager.free) == 16
+
+
+def test_threshold_branch_commits_a_block_in_one_pass():
+    model = ScriptedModel(peak=30.0)                         # every position above 0.9
+    eng = _engine(model)
+    s = eng.add_request(list(range(100)), SamplingParams(max_new_tokens=96, ignore_eos=True, transfer_count=4))
+    eng.generate()
+    assert len(model.calls) == 3 * 2                         # one denoising pass + one caching pass per block
+    assert s.completion_token_ids == [10 + p for p in range(32)] * 3
+
+
+def test_runner_tensors_follow_the_reference_layout():
+    model = ScriptedModel()
+    eng = _engine(model, shuffle_pages_seed=1)
+    sp = SamplingParams(max_new_tokens=32, ignore_eos=True, transfer_count=4)
+    s1 = eng.add_request(list(range(250)), sp)               # crosses a page when the block is appended
+    s2 = eng.add_request(list(range(10)), sp)
+    eng.step()
+    pre = model.calls[0]
+    assert pre["cu"].tolist() == [0, 282, 324]               # prompt + 32 mask tokens per sequence
+    assert pre["positions"].tolist() == list(range(282)) + list(range(42))
+    t1, t2 = list(s1.block_table), list(s2.block_table)
+    want = oracle.get_slots(t1, 0, 250) + [-1] * 32 + oracle.get_slots(t2, 0, 10) + [-1] * 32
+    assert pre["slots"].tolist() == want                     # the uncommitted block is not stored in prefill
+    eng.step()
+    dec = model.calls[1]
+    assert len(s1.block_table) == 2 and len(s2.block_table) == 1      # 250 + 32 > 256 -> second page
+    assert dec["ctx_lens"].tolist() == [282, 42]
+    assert dec["positions"].tolist() == [list(range(250, 282)), list(range(10, 42))]
+    assert dec["slots"].tolist() == [oracle.get_slots(s1.block_table, 250, 282), oracle.get_slots(s2.block_table, 10, 42)]
+    assert dec["tables"].tolist() == [s1.block_table, s2.block_table + [-1]]
+
+
+def test_stop_token_finishes_a_sequence():
+    model = ScriptedModel(peak=30.0)
+    eng = _engine(model)
+    s = eng.add_request(list(range(5)), SamplingParams(max_new_tokens=320, stop_token_ids=[10 + 7], transfer_count=4))
+    eng.generate()
+    assert s.num_completion_tokens == 32 and s.status == SequenceStatus.FINISHED
