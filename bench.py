@@ -258,7 +258,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
-    ap.add_argument("--only", default="", help="comma list of legs to run: step,store,paged,unmask,decode (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,decode (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -273,6 +273,16 @@ def main():
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
     result_ops = {}
+
+    # A plain 1 GiB device copy: the yardstick against which FETCH_SIZE / WRITE_SIZE counter
+    # readings of the kernels below are scaled when this command runs under rocprofv3 --pmc.
+    if want("calib"):
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     # ---------------- config 3: the step (store + staircase attention) -----------------------------
     log("[bench] building config 3 inputs")
@@ -417,6 +427,13 @@ def main():
         except Exception as e:  # the side numbers are informative only
             cpu["other_ops"] = {"error": str(e)}
 
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
+    tfile = ROOT / "profiles" / "traffic.json"
+    if tfile.exists():
+        measured = json.loads(tfile.read_text())
+        for name, op in result_ops.items():
+            if name in measured:
+                op["roofline"]["traffic"] = measured[name]
     value = work3["flops"] / ms_step / 1e9 if ms_step == ms_step else None
     line = {
         "metric": "staircase-attn TFLOP/s (%MFMA peak) + block-diffusion decode tokens/s, 1 GPU",

@@ -16,8 +16,14 @@
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kUnroll = 4;               // 16-byte loads in flight per lane
+#ifndef MDX_UNMASK_THREADS
+#define MDX_UNMASK_THREADS 256
+#endif
+#ifndef MDX_UNMASK_UNROLL
+#define MDX_UNMASK_UNROLL 4
+#endif
+constexpr int kThreads = MDX_UNMASK_THREADS;
+constexpr int kUnroll = MDX_UNMASK_UNROLL;   // 16-byte loads in flight per lane
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -3.0e38f;      // finite stand-in for -inf: keeps (m - m) away from inf - inf
 constexpr int kNoIndex = 0x7fffffff;
@@ -270,10 +276,13 @@ __global__ __launch_bounds__(kThreads) void confidence_finalize_kernel(
     }
 }
 
-// One workgroup per sequence; lane p owns block position p.
+// One workgroup per sequence; lane p owns block position p.  With FROM_PARTIALS the row splits
+// of the vocabulary pass are merged here (and x0 / x0_p written), saving a launch.
 constexpr int kMaxBlockLen = 1024;
+template <bool FROM_PARTIALS>
 __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
-    const int64_t* __restrict__ x0, const float* __restrict__ x0_p, int64_t* __restrict__ tokens,
+    int64_t* __restrict__ x0, float* __restrict__ x0_p, int64_t* __restrict__ tokens,
+    const Partial* __restrict__ partials, int nsplit, const float* __restrict__ temperatures,
     int64_t mask_token_id, float threshold, int k,
     uint8_t* __restrict__ transfer, int32_t* __restrict__ count, int block_len)
 {
@@ -285,8 +294,24 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
     const int64_t at = (int64_t)b * block_len + p;
     if (p == 0) { n_hi = 0; n_masked = 0; n_commit = 0; }
     __syncthreads();
+    int64_t pick = 0;
+    float pick_p = 0.f;
+    if (on) {
+        if (FROM_PARTIALS) {
+            const float c = kLog2e / (temperatures ? temperatures[b] : 1.0f);
+            Partial r = partials[at * nsplit];
+            for (int s = 1; s < nsplit; ++s) combine(r, partials[at * nsplit + s], c, false);
+            pick = r.idx;
+            pick_p = 1.0f / r.s;
+            x0[at] = pick;
+            x0_p[at] = pick_p;
+        } else {
+            pick = x0[at];
+            pick_p = x0_p[at];
+        }
+    }
     const bool masked = on && tokens[at] == mask_token_id;
-    const float conf = masked ? x0_p[at] : -INFINITY;
+    const float conf = masked ? pick_p : -INFINITY;
     const bool hi = conf > threshold;
     if (on) conf_s[p] = conf;
     if (hi) atomicAdd(&n_hi, 1);
@@ -309,7 +334,7 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
     if (on) {
         transfer[at] = commit ? 1 : 0;
         if (commit) {
-            tokens[at] = x0[at];
+            tokens[at] = pick;
             atomicAdd(&n_commit, 1);
         }
     }
@@ -317,10 +342,10 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
     if (p == 0) count[b] = n_commit;
 }
 
-// Splits per row so that small batches still fill the chip: target >= ~2 waves of workgroups
+// Splits per row so that small batches still fill the chip: target >= 4 workgroups per CU
 // while keeping at least 32 KiB of logits per workgroup.
 int pick_nsplit(int64_t rows, int64_t vocab) {
-    const int64_t target = 2048;
+    const int64_t target = 1024;
     int64_t n = (target + rows - 1) / rows;
     const int64_t max_by_size = vocab / 16384 > 0 ? vocab / 16384 : 1;
     if (n > max_by_size) n = max_by_size;
@@ -332,7 +357,7 @@ int pick_nsplit(int64_t rows, int64_t vocab) {
 template <typename T>
 int launch_confidence(const void* logits, int64_t row_stride, const float* temperatures, int rows_per_temp,
                       const float* noise, int64_t noise_row_stride, int64_t* x0, float* x0_p,
-                      int64_t rows, int64_t vocab, int nsplit, Partial* partials, hipStream_t stream)
+                      int64_t rows, int64_t vocab, int nsplit, Partial* partials, bool finalize, hipStream_t stream)
 {
     const dim3 grid((unsigned)rows, (unsigned)nsplit);
     if (noise)
@@ -342,7 +367,7 @@ int launch_confidence(const void* logits, int64_t row_stride, const float* tempe
         confidence_argmax_kernel<T, false><<<grid, kThreads, 0, stream>>>(
             (const T*)logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, vocab, nsplit, partials, x0, x0_p);
     int rc = mdx::check_launch("confidence_argmax");
-    if (rc != MDX_OK || nsplit == 1) return rc;
+    if (rc != MDX_OK || nsplit == 1 || !finalize) return rc;
     const unsigned fgrid = (unsigned)((rows + kThreads - 1) / kThreads);
     if (noise)
         confidence_finalize_kernel<true><<<fgrid, kThreads, 0, stream>>>(partials, nsplit, temperatures, rows_per_temp, rows, x0, x0_p);
@@ -359,14 +384,16 @@ extern "C" int64_t mdx_confidence_argmax_workspace_bytes(int64_t rows, int64_t v
     return nsplit > 1 ? rows * nsplit * (int64_t)sizeof(Partial) : 0;
 }
 
-extern "C" int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
-                                     const float* temperatures, int32_t rows_per_temp,
-                                     const float* noise, int64_t noise_row_stride,
-                                     int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
-                                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream_)
+namespace {
+
+int confidence_pass(const void* logits, int64_t row_stride, int32_t dtype,
+                    const float* temperatures, int32_t rows_per_temp,
+                    const float* noise, int64_t noise_row_stride,
+                    int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
+                    void* workspace, int64_t workspace_bytes, bool finalize, int* nsplit_out, hipStream_t stream)
 {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(rows >= 0 && vocab >= 0, MDX_EINVAL, "confidence_argmax: negative size");
+    if (nsplit_out) *nsplit_out = 1;
     if (rows == 0) return MDX_OK;
     MDX_REQUIRE(vocab > 0, MDX_EINVAL, "confidence_argmax: empty vocabulary");
     MDX_REQUIRE(logits && x0 && x0_p, MDX_EINVAL, "confidence_argmax: null pointer");
@@ -378,16 +405,29 @@ extern "C" int mdx_confidence_argmax(const void* logits, int64_t row_stride, int
     const int esz = dtype == MDX_F32 ? 4 : 2;
     MDX_REQUIRE((reinterpret_cast<uintptr_t>(logits) % esz) == 0, MDX_EUNSUPPORTED, "confidence_argmax: logits not element-aligned");
     const int nsplit = pick_nsplit(rows, vocab);
+    if (nsplit_out) *nsplit_out = nsplit;
     const int64_t need = nsplit > 1 ? rows * nsplit * (int64_t)sizeof(Partial) : 0;
     MDX_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), MDX_EWORKSPACE,
                 "confidence_argmax: workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
     Partial* partials = static_cast<Partial*>(workspace);
     switch (dtype) {
-        case MDX_BF16: return launch_confidence<__bf16>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
-        case MDX_F16:  return launch_confidence<__half>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
-        case MDX_F32:  return launch_confidence<float>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, stream);
+        case MDX_BF16: return launch_confidence<__bf16>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
+        case MDX_F16:  return launch_confidence<__half>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
+        case MDX_F32:  return launch_confidence<float>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
         default: return mdx::fail(MDX_EUNSUPPORTED, "confidence_argmax: dtype %d", dtype);
     }
+}
+
+}  // namespace
+
+extern "C" int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
+                                     const float* temperatures, int32_t rows_per_temp,
+                                     const float* noise, int64_t noise_row_stride,
+                                     int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
+                                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    return confidence_pass(logits, row_stride, dtype, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p,
+                           rows, vocab, workspace, workspace_bytes, true, nullptr, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t* tokens,
@@ -402,7 +442,8 @@ extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "select_transfer: block_len %d > %d", block_len, kMaxBlockLen);
     MDX_REQUIRE(k >= 1, MDX_EINVAL, "select_transfer: k %d < 1", k);
     const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
-    select_transfer_kernel<<<(unsigned)bs, threads, 0, stream>>>(x0, x0_p, tokens, mask_token_id, threshold, k, transfer, count, block_len);
+    select_transfer_kernel<false><<<(unsigned)bs, threads, 0, stream>>>(
+        const_cast<int64_t*>(x0), const_cast<float*>(x0_p), tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
     return mdx::check_launch("select_transfer");
 }
 
@@ -411,15 +452,25 @@ extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t d
                                int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
                                int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
                                int32_t bs, int32_t block_len, int64_t vocab,
-                               void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+                               void* workspace, int64_t workspace_bytes, mdx_stream_t stream_)
 {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && block_len >= 0, MDX_EINVAL, "unmask_step: negative size");
     MDX_REQUIRE(k >= 1, MDX_EINVAL, "unmask_step: k %d < 1", k);
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "unmask_step: block_len %d > %d", block_len, kMaxBlockLen);
     if (bs == 0 || block_len == 0) return MDX_OK;
     MDX_REQUIRE(tokens && transfer && count, MDX_EINVAL, "unmask_step: null pointer");
-    int rc = mdx_confidence_argmax(logits, row_stride, dtype, temperatures, block_len, noise, noise_row_stride,
-                                   x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, stream);
+    // Without noise the selection kernel merges the row splits itself (one launch fewer).
+    int nsplit = 1;
+    int rc = confidence_pass(logits, row_stride, dtype, temperatures, block_len, noise, noise_row_stride,
+                             x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, noise != nullptr, &nsplit, stream);
     if (rc != MDX_OK) return rc;
-    return mdx_select_transfer(x0, x0_p, tokens, mask_token_id, threshold, k, transfer, count, bs, block_len, stream);
+    const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
+    if (nsplit > 1 && !noise)
+        select_transfer_kernel<true><<<(unsigned)bs, threads, 0, stream>>>(
+            x0, x0_p, tokens, static_cast<const Partial*>(workspace), nsplit, temperatures, mask_token_id, threshold, k, transfer, count, block_len);
+    else
+        select_transfer_kernel<false><<<(unsigned)bs, threads, 0, stream>>>(
+            x0, x0_p, tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
+    return mdx::check_launch("select_transfer");
 }
