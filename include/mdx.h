@@ -175,6 +175,32 @@ int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
                     int32_t bs, int32_t block_len, int64_t vocab,
                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
 
+/*
+ * Fused producer of the attention inputs for one decoder layer: per-head RMSNorm of q and k,
+ * rotary embedding, and the KV-cache store, in one pass over the fused QKV projection output --
+ * replaces the chain q_norm / k_norm / rotary_emb / store_kvcache of
+ * engines/nano_dvlm/nanovllm/models/sdar.py:79-83 (layers/layernorm.py:16-26,
+ * layers/rotary_embedding.py:6-14,37-48, layers/sdar_attention.py:37-38).
+ *
+ * qkv [n_tokens, (Hq + 2 Hkv) * d] (row stride in elements; heads laid out q | k | v);
+ * q_weight, k_weight [d]; cos_table, sin_table [max_positions, d/2] fp32; positions [n_tokens]
+ * int64.  Writes q_out [n_tokens, Hq, d] and, if non-null, k_out [n_tokens, Hkv, d] (the
+ * rotated k the prefill attention reads), and, if the caches are given, the rotated k row and
+ * the raw v row of token i into slot slot_mapping[i] (-1 and out-of-range slots skipped) of
+ * k_cache / v_cache [num_slots, Hkv, d].  v itself stays where it is (a view of qkv).
+ * Rounding follows the reference: normalise in fp32, round to bf16, multiply by the weight
+ * in bf16, rotate in fp32, round once.  Supported: d == 128, MDX_BF16.
+ */
+int mdx_qk_norm_rope_store(const void* qkv, int64_t qkv_row_stride,
+                           const void* q_weight, const void* k_weight, float eps,
+                           const float* cos_table, const float* sin_table, int64_t max_positions,
+                           const int64_t* positions,
+                           void* q_out, int64_t q_out_row_stride,
+                           void* k_out, int64_t k_out_row_stride,
+                           void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t num_slots,
+                           int64_t n_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                           int32_t dtype, mdx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,8 @@ SIGNATURES = {
     "mdx_confidence_argmax_workspace_bytes": (c_int64, [_I64, _I64]),
     "mdx_confidence_argmax": (c_int32, [_P, _I64, _I32, _P, _I32, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _P]),
     "mdx_select_transfer": (c_int32, [_P, _P, _P, _I64, _F, _I32, _P, _P, _I32, _I32, _P]),
+    "mdx_qk_norm_rope_store": (c_int32, [_P, _I64, _P, _P, _F, _P, _P, _I64, _P, _P, _I64, _P, _I64, _P, _P, _P, _I64,
+                                         _I64, _I32, _I32, _I32, _I32, _P]),
     "mdx_unmask_step": (c_int32, [_P, _I64, _I32, _P, _P, _I64, _P, _I64, _F, _I32, _P, _P, _P, _P,
                                   _I32, _I32, _I64, _P, _I64, _P]),
 }

@@ -30,7 +30,7 @@ from torch import nn
 
 from .context import get_context, reset_context, set_context
 from .layers import Attention
-from .ops import unmask_step
+from .ops import flash_attn_with_kvcache, qk_norm_rope_store, sparse_attn_varlen, unmask_step
 
 PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
 
@@ -169,6 +169,7 @@ class DecoderConfig:
     max_position: int = 8192
     block_size: int = 32
     mask_token_id: int = 151669
+    fused_qk_rope_store: bool = True    # one libmdx launch for q/k norm + RoPE + KV store (else stock ops)
 
 
 def _rms(x, w, eps):
@@ -190,7 +191,7 @@ class DecoderLayer(nn.Module):
         self.post_attention_layernorm = nn.Parameter(torch.ones(c.hidden_size))
         self.attn = Attention(c.num_heads, c.head_dim, c.head_dim ** -0.5, c.num_kv_heads)
 
-    def forward(self, positions, x, residual, cos, sin):
+    def forward(self, positions, x, residual, cos, sin, cos_table=None, sin_table=None):
         c = self.c
         if residual is None:                               # sdar.py:147-150
             residual = x
@@ -199,19 +200,40 @@ class DecoderLayer(nn.Module):
             residual = x + residual
             h = _rms(residual, self.input_layernorm, c.rms_norm_eps)
         qkv = F.linear(h, self.qkv_proj)
-        q_size, kv_size = c.num_heads * c.head_dim, c.num_kv_heads * c.head_dim
-        q, k, v = qkv.split([q_size, kv_size, kv_size], dim=-1)
-        shape = (*positions.shape, -1, c.head_dim)
-        q, k, v = q.view(shape), k.view(shape), v.view(shape)   # v stays a strided view of qkv
-        q = _rms(q, self.q_norm, c.rms_norm_eps)
-        k = _rms(k, self.k_norm, c.rms_norm_eps)
-        q, k = _rope(q, cos, sin), _rope(k, cos, sin)
-        o = self.attn(q, k, v)
+        if c.fused_qk_rope_store:
+            o = self._attend_fused(qkv, positions, cos_table, sin_table)
+        else:
+            q_size, kv_size = c.num_heads * c.head_dim, c.num_kv_heads * c.head_dim
+            q, k, v = qkv.split([q_size, kv_size, kv_size], dim=-1)
+            shape = (*positions.shape, -1, c.head_dim)
+            q, k, v = q.view(shape), k.view(shape), v.view(shape)   # v stays a strided view of qkv
+            q = _rms(q, self.q_norm, c.rms_norm_eps)
+            k = _rms(k, self.k_norm, c.rms_norm_eps)
+            q, k = _rope(q, cos, sin), _rope(k, cos, sin)
+            o = self.attn(q, k, v)
         x = F.linear(o, self.o_proj)
         residual = x + residual
         h = _rms(residual, self.post_attention_layernorm, c.rms_norm_eps)
         gate, up = F.linear(h, self.gate_up_proj).chunk(2, dim=-1)
         return F.linear(F.silu(gate) * up, self.down_proj), residual
+
+
+    def _attend_fused(self, qkv, positions, cos_table, sin_table):
+        """sdar.py:79-83 + sdar_attention.py:34-57 with the q/k norm, RoPE and cache store done by
+        one libmdx launch; the attention calls are the same two as in `Attention.forward`."""
+        c, attn, ctx = self.c, self.attn, get_context()
+        have_cache = attn.k_cache.numel() > 0
+        q, k, v = qk_norm_rope_store(qkv, self.q_norm, self.k_norm, c.rms_norm_eps, cos_table, sin_table, positions,
+                                     c.num_heads, c.num_kv_heads, c.head_dim,
+                                     attn.k_cache if have_cache else None, attn.v_cache if have_cache else None,
+                                     ctx.slot_mapping if have_cache else None, want_k=ctx.is_prefill)
+        if ctx.is_prefill:
+            o = sparse_attn_varlen(q, k, v, cu_seqlens_q=ctx.cu_seqlens_q, cu_seqlens_k=ctx.cu_seqlens_k,
+                                   staircase_size=ctx.block_size, max_seqlen=ctx.max_seqlen_k or None, softmax_scale=attn.scale)
+            return o.flatten(1)
+        o = flash_attn_with_kvcache(q, attn.k_cache, attn.v_cache, cache_seqlens=ctx.context_lens,
+                                    block_table=ctx.block_tables, softmax_scale=attn.scale, causal=False)
+        return o.flatten(2)
 
 
 def _rope(x, cos, sin):                                    # rotary_embedding.py:6-14
@@ -245,11 +267,13 @@ class Decoder(nn.Module):
 
     @torch.inference_mode()
     def forward(self, inputs_embeds, positions):
-        cos = self.cos[positions].unsqueeze(-2)
-        sin = self.sin[positions].unsqueeze(-2)
+        cos = sin = None
+        if not self.c.fused_qk_rope_store:
+            cos = self.cos[positions].unsqueeze(-2)
+            sin = self.sin[positions].unsqueeze(-2)
         x, residual = inputs_embeds, None
         for layer in self.layers:
-            x, residual = layer(positions, x, residual, cos, sin)
+            x, residual = layer(positions, x, residual, cos, sin, self.cos, self.sin)
         return _rms(x + residual, self.norm, self.c.rms_norm_eps)
 
     @torch.inference_mode()

@@ -64,6 +64,46 @@ def store_kvcache_maybe4d(k, v, k_cache, v_cache, slot_mapping) -> None:
     store_kvcache(k, v, k_cache, v_cache, slot_mapping)
 
 
+def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float,
+                       cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                       num_q_heads: int, num_kv_heads: int, head_dim: int,
+                       k_cache: torch.Tensor | None = None, v_cache: torch.Tensor | None = None,
+                       slot_mapping: torch.Tensor | None = None, want_k: bool = True):
+    """One launch for nanovllm/models/sdar.py:79-83 plus the cache store: qkv [..., (Hq+2Hkv)*d]
+    -> (q [..., Hq, d], k [..., Hkv, d] or None, v view [..., Hkv, d]); rotated k and raw v are
+    written to the caches at slot_mapping when caches are given.  cos/sin: fp32 [max_pos, d/2]."""
+    _need_gpu(qkv, q_weight, k_weight, cos, sin, positions, k_cache, v_cache, slot_mapping)
+    lead = qkv.shape[:-1]
+    width = (num_q_heads + 2 * num_kv_heads) * head_dim
+    assert qkv.shape[-1] == width and qkv.stride(-1) == 1
+    q2 = qkv.reshape(-1, width)
+    n = q2.shape[0]
+    pos = positions.reshape(-1)
+    assert pos.numel() == n and pos.dtype == torch.int64 and cos.dtype == torch.float32 and sin.dtype == torch.float32
+    pos = pos if pos.is_contiguous() else pos.contiguous()
+    q = torch.empty((n, num_q_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    k = torch.empty((n, num_kv_heads, head_dim), dtype=qkv.dtype, device=qkv.device) if want_k else None
+    slots = None
+    num_slots = 0
+    if k_cache is not None and k_cache.numel():
+        assert k_cache.is_contiguous() and v_cache.is_contiguous()
+        slots = _i32(slot_mapping.reshape(-1), "slot_mapping")
+        assert slots.numel() == n
+        num_slots = k_cache.numel() // (num_kv_heads * head_dim)
+    else:
+        k_cache = v_cache = None
+    rc = _lib.lib().mdx_qk_norm_rope_store(
+        q2.data_ptr(), q2.stride(0), q_weight.data_ptr(), k_weight.data_ptr(), float(eps),
+        cos.data_ptr(), sin.data_ptr(), cos.shape[0], pos.data_ptr(),
+        q.data_ptr(), q.stride(0), k.data_ptr() if k is not None else None, k.stride(0) if k is not None else 0,
+        k_cache.data_ptr() if k_cache is not None else None, v_cache.data_ptr() if v_cache is not None else None,
+        slots.data_ptr() if slots is not None else None, num_slots,
+        n, num_q_heads, num_kv_heads, head_dim, _DTYPES[qkv.dtype], _stream(qkv))
+    check(rc, "qk_norm_rope_store")
+    v = qkv[..., (num_q_heads + num_kv_heads) * head_dim:].unflatten(-1, (num_kv_heads, head_dim))   # strided view
+    return q.view(*lead, num_q_heads, head_dim), None if k is None else k.view(*lead, num_kv_heads, head_dim), v
+
+
 # --------------------------------------------------------------------------- staircase prefill
 def sparse_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
                        cu_seqlens_k: torch.Tensor, staircase_size: int = 4, *, max_seqlen: int | None = None,

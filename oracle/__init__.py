@@ -29,6 +29,8 @@ confidence_argmax           torch.softmax / torch.argmax, fp64 explicit sums
 select_transfer             torch.topk on tie-free inputs, brute force over all
                             subsets on 6 positions, counting invariants
 slot_of / get_slots         brute force token-by-token formula
+rms_norm_ref / rope_ref     unit RMS after norm, F.rms_norm, rotation preserves pair norms,
+                            position 0 is the identity, complex-multiplication form
 dense_forward               built from the pinned attention oracle and plain matmuls; its mask
                             and SDPA are the functions above
 ==========================  =====================================================
@@ -47,3 +49,4 @@ from .kvstore import store_kvcache  # noqa: F401
 from .unmask import confidence_argmax, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
 from .slots import slot_of, get_slots  # noqa: F401
 from .engine import dense_forward, expected_passes  # noqa: F401
+from .fused import qk_norm_rope, rms_norm_ref, rope_ref  # noqa: F401
