@@ -1,8 +1,8 @@
 // Wavefront-level building block shared by the two attention kernels
 // (staircase block-prefill and paged single-block decode), head_dim 128, bf16.
 //
-// One wavefront owns 32 query rows (one MFMA column tile) of one query head
-// and walks over keys 32 at a time:
+// One wavefront owns 32 query rows (one MFMA column tile) of NH query heads that share a KV
+// head and walks over keys 32 at a time:
 //
 //   S^T[key, query]  = K[key, :] . Q[query, :]      v_mfma_f32_32x32x16_bf16, A = K (LDS), B = Q^T (registers)
 //   online softmax   per query = per LANE            row max / sum live in the lane, one permlane32_swap per step
@@ -64,42 +64,49 @@ __device__ __forceinline__ float both_halves_sum(float x) {
 typedef __attribute__((address_space(3))) char lds_char;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
-// Running state of one wavefront: one head x 32 queries.
+// Running state of one wavefront: NH heads x 32 queries.  With NH = 2 the two query heads of a
+// grouped-query pair share every K and V fragment fetched from LDS (half the LDS bytes per MFMA).
+template <int NH>
 struct WaveState {
-    float m;                // running max, in log2 units (score * scale * log2 e); same in both half-waves
-    float l;                // running sum of this half-wave's keys only
-    f32x16 o[4];            // O^T: 4 tiles of 32 d-rows x 32 queries
+    float m[NH];            // running max, in log2 units (score * scale * log2 e); same in both half-waves
+    float l[NH];            // running sum of this half-wave's keys only
+    f32x16 o[NH][4];        // O^T: 4 tiles of 32 d-rows x 32 queries
     __device__ __forceinline__ void init() {
-        m = kMinusBig;
-        l = 0.f;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int h = 0; h < NH; ++h) {
+            m[h] = kMinusBig;
+            l[h] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) o[t][i] = 0.f;
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[h][t][i] = 0.f;
+        }
     }
 };
 
 // The three phases of one online-softmax step over NSUB*32 keys held in LDS rows
-// n0 .. n0+NSUB*32-1 of tiles with row pitch kLdsPitch.  They are separate so that the
-// wavefronts sharing a SIMD can run them out of phase (one in MFMA while the other is in
-// its softmax).
+// n0 .. n0+NSUB*32-1 of tiles with row pitch kLdsPitch.
 
-// S^T = K Q^T.  q[ks] are the B-operand fragments of Q^T for d = 16ks .. 16ks+15.
-template <int NSUB>
-__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8 (&q)[8], f32x16 (&s)[NSUB], int lane)
+// S^T = K Q^T.  q[h][ks] are the B-operand fragments of Q^T for d = 16ks .. 16ks+15.
+template <int NH, int NSUB>
+__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8 (&q)[NH][8], f32x16 (&s)[NH][NSUB], int lane)
 {
     const int H = lane >> 5, r = lane & 31;
 #pragma unroll
-    for (int u = 0; u < NSUB; ++u)
+    for (int h = 0; h < NH; ++h)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[u][i] = 0.f;
+        for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[h][u][i] = 0.f;
     const char* kbase = lds_k + (n0 + key_of_mfma_row(r)) * kLdsPitch + H * 16;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kbase + u * 32 * kLdsPitch + ks * 32);
-            s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[ks], s[u], 0, 0, 0);
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+                s[h][u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[h][ks], s[h][u], 0, 0, 0);
         }
     }
 }
@@ -107,62 +114,65 @@ __device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8
 // Online softmax, per lane = per query.  c = softmax scale * log2(e) (> 0).
 // MASK: keys with absolute index outside [key_lo, key_hi) are excluded; key_abs0 is the
 // absolute index of LDS row n0; key_hi may differ per lane (per query), key_lo is uniform.
-// Produces the bf16 B-operand fragments p[u][t] of P^T and updates m, l and (when the
+// Produces the bf16 B-operand fragments p[h][u][t] of P^T and updates m, l and (when the
 // running max moves) rescales O.
-template <int NSUB, bool MASK>
-__device__ __forceinline__ void softmax_phase(f32x16 (&s)[NSUB], bf16x8 (&p)[2][2], WaveState& st, float c, int lane,
-                                              int key_abs0, int key_lo, int key_hi)
+template <int NH, int NSUB, bool MASK>
+__device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], bf16x8 (&p)[NH][NSUB][2], WaveState<NH>& st, float c,
+                                              int lane, int key_abs0, int key_lo, int key_hi)
 {
     const int H = lane >> 5;
-    if (MASK) {
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+        if (MASK) {
+#pragma unroll
+            for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int key = key_abs0 + 32 * u + key_of_reg(i, H);
+                    s[h][u][i] = (key >= key_lo && key < key_hi) ? s[h][u][i] : -INFINITY;
+                }
+        }
+        float mx = s[h][0][0];
 #pragma unroll
         for (int u = 0; u < NSUB; ++u)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int key = key_abs0 + 32 * u + key_of_reg(i, H);
-                s[u][i] = (key >= key_lo && key < key_hi) ? s[u][i] : -INFINITY;
-            }
+            for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[h][u][i]);
+        mx = other_half_max(mx);
+        // Lazy rescale: the running max only moves when some query's new max exceeds it by more
+        // than kMaxSlack (log2 units).  Until then probabilities are taken relative to the stale
+        // max (at most 2^kMaxSlack, harmless in fp32/bf16) and O, l need no rescaling; the final
+        // O / l is unchanged because numerator and denominator share the same reference.
+        const float m_cand = fmaxf(st.m[h], mx * c);
+        const bool moved = __any(m_cand > st.m[h] + kMaxSlack);         // wave-uniform
+        const float m_new = moved ? m_cand : st.m[h];
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float e = __builtin_amdgcn_exp2f(fmaf(s[h][u][8 * t + j], c, -m_new));
+                    sum += e;
+                    p[h][u][t][j] = (__bf16)e;
+                }
+        if (moved) {
+            const float alpha = __builtin_amdgcn_exp2f(st.m[h] - m_new);
+            st.l[h] *= alpha;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) st.o[h][t][i] *= alpha;
+            st.m[h] = m_new;
+        }
+        st.l[h] += sum;
     }
-    float mx = s[0][0];
-#pragma unroll
-    for (int u = 0; u < NSUB; ++u)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[u][i]);
-    mx = other_half_max(mx);
-    // Lazy rescale: the running max only moves when some query's new max exceeds it by more
-    // than kMaxSlack (log2 units).  Until then probabilities are taken relative to the stale
-    // max (at most 2^kMaxSlack, harmless in fp32/bf16) and O, l need no rescaling; the final
-    // O / l is unchanged because numerator and denominator share the same reference.
-    const float m_cand = fmaxf(st.m, mx * c);
-    const bool moved = __any(m_cand > st.m + kMaxSlack);            // wave-uniform
-    const float m_new = moved ? m_cand : st.m;
-    float sum = 0.f;
-#pragma unroll
-    for (int u = 0; u < NSUB; ++u)
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float e = __builtin_amdgcn_exp2f(fmaf(s[u][8 * t + j], c, -m_new));
-                sum += e;
-                p[u][t][j] = (__bf16)e;
-            }
-    if (moved) {
-        const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);
-        st.l *= alpha;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) st.o[t][i] *= alpha;
-        st.m = m_new;
-    }
-    st.l += sum;
 }
 
 // O^T += V^T P^T.  The lane supplies the row address for the transposing read:
 // row 4*(i'/4) + 2H (+q), d chunk i'%4, with i' = lane % 16.
-template <int NSUB>
-__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const bf16x8 (&p)[2][2], WaveState& st, int lane)
+template <int NH, int NSUB>
+__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const bf16x8 (&p)[NH][NSUB][2], WaveState<NH>& st, int lane)
 {
     const int H = lane >> 5, ip = lane & 15, gi = (lane >> 4) & 1;
     const lds_char* vbase = (const lds_char*)lds_v + (n0 + 4 * (ip >> 2) + 2 * H) * kLdsPitch + (gi * 16 + (ip & 3) * 4) * 2;
@@ -176,20 +186,23 @@ __device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const bf16x8
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a);
                 const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + kLdsPitch));
                 const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                st.o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), p[u][t], st.o[dt], 0, 0, 0);
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+#pragma unroll
+                for (int h = 0; h < NH; ++h)
+                    st.o[h][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p[h][u][t], st.o[h][dt], 0, 0, 0);
             }
 }
 
 // All three phases back to back.
-template <int NSUB, bool MASK>
-__device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, int n0, const bf16x8 (&q)[8],
-                                          WaveState& st, float c, int lane, int key_abs0, int key_lo, int key_hi)
+template <int NH, int NSUB, bool MASK>
+__device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, int n0, const bf16x8 (&q)[NH][8],
+                                          WaveState<NH>& st, float c, int lane, int key_abs0, int key_lo, int key_hi)
 {
-    f32x16 s[NSUB];
-    bf16x8 p[2][2];
-    qk_phase<NSUB>(lds_k, n0, q, s, lane);
-    softmax_phase<NSUB, MASK>(s, p, st, c, lane, key_abs0, key_lo, key_hi);
-    pv_phase<NSUB>(lds_v, n0, p, st, lane);
+    f32x16 s[NH][NSUB];
+    bf16x8 p[NH][NSUB][2];
+    qk_phase<NH, NSUB>(lds_k, n0, q, s, lane);
+    softmax_phase<NH, NSUB, MASK>(s, p, st, c, lane, key_abs0, key_lo, key_hi);
+    pv_phase<NH, NSUB>(lds_v, n0, p, st, lane);
 }
 
 // d index held by accumulator register i of O^T tile dt in half-wave H.

@@ -103,10 +103,10 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
     const int kvh = (hg * HPW) / P.heads_per_kv;
 
     const bool row_ok = r < P.sq;
-    bf16x8 q[8];
-    load_q(q, row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H);
+    bf16x8 q[1][8];
+    load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H);
 
-    WaveState st;
+    WaveState<1> st;
     st.init();
 
     const int32_t* bt = P.block_table + (int64_t)b * P.bt_stride;
@@ -156,9 +156,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         // keys of an invalid page are excluded (not merely zeroed): the owning wavefront skips them
         if ((tile_pass_ok[t & 1] >> (2 * kw)) & 1u) {
             if (key0 + 32 <= key_end)
-                attn_step<1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<1, 1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
             else
-                attn_step<1, true>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<1, 1, true>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
         }
     };
 
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
     }
 
     // ---- merge the KW key-slice states of each head (tree through LDS) ----------------------
-    st.l = both_halves_sum(st.l);          // a state is now (m, l, O) per query
+    st.l[0] = both_halves_sum(st.l[0]);          // a state is now (m, l, O) per query
     // Exchange layout per sending wavefront: O as [4][16][64 lanes] floats, then m, l as [64].
     constexpr int kStateFloats = 4 * 16 * 64 + 2 * 64;
     static_assert(HPW * (KW / 2) * kStateFloats * 4 <= (int)sizeof(lds), "merge buffer exceeds the tile region");
@@ -203,23 +203,23 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = st.o[t][i];
-        dst[4 * 16 * 64 + lane] = st.m;
-        dst[4 * 16 * 64 + 64 + lane] = st.l;
+            for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = st.o[0][t][i];
+        dst[4 * 16 * 64 + lane] = st.m[0];
+        dst[4 * 16 * 64 + 64 + lane] = st.l[0];
     };
     auto recv = [&](int slot) {
         const float* src = xch + slot * kStateFloats;
         const float m2 = src[4 * 16 * 64 + lane];
         const float l2 = src[4 * 16 * 64 + 64 + lane];
-        const float M = fmaxf(st.m, m2);
-        const float a1 = __builtin_amdgcn_exp2f(st.m - M), a2 = __builtin_amdgcn_exp2f(m2 - M);
-        st.l = st.l * a1 + l2 * a2;
-        st.m = M;
+        const float M = fmaxf(st.m[0], m2);
+        const float a1 = __builtin_amdgcn_exp2f(st.m[0] - M), a2 = __builtin_amdgcn_exp2f(m2 - M);
+        st.l[0] = st.l[0] * a1 + l2 * a2;
+        st.m[0] = M;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i)
-                st.o[t][i] = st.o[t][i] * a1 + src[(t * 16 + i) * 64 + lane] * a2;
+                st.o[0][t][i] = st.o[0][t][i] * a1 + src[(t * 16 + i) * 64 + lane] * a2;
     };
     // (the loop's last barrier already separates the tile reads from these writes)
 #pragma unroll
@@ -233,7 +233,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
 
     // ---- output ---------------------------------------------------------------
     if (n_valid_splits == 1) {
-        const float inv = 1.0f / st.l;
+        const float inv = 1.0f / st.l[0];
         __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)r * P.o_ss + (int64_t)head * P.o_sh;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
                 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
                 bf16x4 out;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[dt][4 * g + e] * inv);
+                for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
                 *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
             }
     } else {
@@ -252,12 +252,12 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float4 out = make_float4(st.o[dt][4 * g], st.o[dt][4 * g + 1], st.o[dt][4 * g + 2], st.o[dt][4 * g + 3]);
+                float4 out = make_float4(st.o[0][dt][4 * g], st.o[0][dt][4 * g + 1], st.o[0][dt][4 * g + 2], st.o[0][dt][4 * g + 3]);
                 *reinterpret_cast<float4*>(po + d_of_reg(dt, 4 * g, H)) = out;
             }
         if (H == 0) {
-            P.part_ml[(slot * 2 + 0) * kMaxSq + r] = st.m;
-            P.part_ml[(slot * 2 + 1) * kMaxSq + r] = st.l;
+            P.part_ml[(slot * 2 + 0) * kMaxSq + r] = st.m[0];
+            P.part_ml[(slot * 2 + 1) * kMaxSq + r] = st.l[0];
         }
     }
 }

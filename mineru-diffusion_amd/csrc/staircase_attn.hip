@@ -112,8 +112,8 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     const int ip = row_w0 + r;                                 // this lane's padded query row
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
-    bf16x8 q[8];
-    load_q(q, row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
+    bf16x8 q[1][8];
+    load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
 
     // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
     const int n_tiles = (wg_hi + kTileKeys - 1) / kTileKeys;
 
-    WaveState st;
+    WaveState<1> st;
     st.init();
 
     // ---- K/V tile pipeline: registers hold tile t+1 while LDS holds tile t (other buffer: t-1) ----
@@ -164,11 +164,11 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         const int key0 = t * kTileKeys;
         if (key0 < wave_hi) {
             if (key0 >= pad && key0 + kTileKeys <= wave_hi_min) {
-                attn_step<2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else if (key0 + 32 < wave_hi) {
-                attn_step<2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else {
-                attn_step<1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             }
         }
         if (t + 1 < n_tiles) {
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 
     // ---- epilogue: O = O^T / l, bf16, 4 consecutive d per store ----
     if (!row_ok) return;
-    const float inv = 1.0f / both_halves_sum(st.l);
+    const float inv = 1.0f / both_halves_sum(st.l[0]);
     __bf16* orow = P.o + tok * P.o_st + (int64_t)head * P.o_sh;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
             typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
             bf16x4 out;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[dt][4 * g + e] * inv);
+            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
             *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
         }
 }
