@@ -428,12 +428,12 @@ def main():
             cpu["other_ops"] = {"error": str(e)}
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
-    tfile = ROOT / "profiles" / "traffic.json"
+    tfile = ROOT / "profiles" / "hbm_traffic_per_call.txt"
     if tfile.exists():
-        measured = json.loads(tfile.read_text())
+        measured = json.loads("".join(l for l in tfile.read_text().splitlines(True) if not l.startswith("#")))
         for name, op in result_ops.items():
             if name in measured:
-                op["roofline"]["traffic"] = measured[name]
+                op["roofline"]["traffic"] = measured[name]["bytes"]
     value = work3["flops"] / ms_step / 1e9 if ms_step == ms_step else None
     line = {
         "metric": "staircase-attn TFLOP/s (%MFMA peak) + block-diffusion decode tokens/s, 1 GPU",
