@@ -64,6 +64,11 @@ __device__ __forceinline__ float both_halves_sum(float x) {
 typedef __attribute__((address_space(3))) char lds_char;
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 
+// 32-bit LDS byte address of a pointer into shared memory (what ds_* instructions take).
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(uintptr_t)(const lds_char*)p;
+}
+
 // Running state of one wavefront: NH heads x 32 queries.  With NH = 2 the two query heads of a
 // grouped-query pair share every K and V fragment fetched from LDS (half the LDS bytes per MFMA).
 template <int NH>

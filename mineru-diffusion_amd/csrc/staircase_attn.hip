@@ -45,26 +45,17 @@ struct StaircaseParams {
     float c;                                                   // scale * log2(e)
 };
 
-__global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const StaircaseParams P)
+// Workgroup -> (sequence b, row group rg) for the j-th (sequence, row group) pair in launch order.
+// Row groups are handed out heaviest-first (the last row group of a sequence attends to the most
+// keys).  The dispatcher deals consecutive workgroups round-robin to XCDs and shader engines and
+// blocks on a full one, so neighbours in launch order must weigh the same: the head slot varies
+// fastest, then the sequences that own a row group at this level, and workgroups that find no
+// work may only sit at the very end of the grid.  With up to 64 sequences each wavefront derives
+// this dense numbering itself (lane b holds sequence b's row-group count, lane r evaluates
+// F(r) = #pairs at level >= r); beyond that the grid is the full (level x sequence) rectangle and
+// absent pairs return at once.  Returns false when there is no such pair.
+__device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j, int lane, int& b, int& rg)
 {
-    __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
-    __shared__ __attribute__((aligned(16))) char lds_vbuf[2][kTileBytes];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int H = lane >> 5, r = lane & 31;
-
-    // ---- workgroup -> (head group, sequence b, row group rg) -----------------------------------
-    // Row groups are handed out heaviest-first (the last row group of a sequence attends to the
-    // most keys).  The dispatcher deals consecutive workgroups round-robin to XCDs and shader
-    // engines and blocks on a full one, so neighbours in launch order must weigh the same:
-    // the head group varies fastest, then the sequences that own a row group at this level, and
-    // workgroups that find no work may only sit at the very end of the grid.  With up to 64
-    // sequences each wavefront derives this dense numbering itself (lane b holds sequence b's
-    // row-group count, lane r evaluates F(r) = #pairs at level >= r); beyond that the grid is the
-    // full (level x sequence) rectangle and absent pairs return at once.
-    const int hslot = blockIdx.x % P.num_q_heads;
-    const int j = blockIdx.x / P.num_q_heads;
-    int b, rg;
     if (P.batch <= 64) {
         int g = 0;                                             // row groups of sequence `lane`
         if (lane < P.batch) {
@@ -83,7 +74,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
             f_level = __builtin_amdgcn_readlane(f, n - 1);
             if (n < 64) break;
         }
-        if (level < 0) return;                                 // past the last pair
+        if (level < 0) return false;                           // past the last pair
         const unsigned long long owners = __ballot(g > level); // sequences that have this row group
         const int nth = j - f_level + __popcll(owners);        // index among them
         const int before = __popcll(owners & ((1ull << lane) - 1ull));
@@ -94,6 +85,21 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         b = j % P.batch;
         rg = P.n_row_groups - 1 - j / P.batch;
     }
+    return true;
+}
+
+__global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const StaircaseParams P)
+{
+    __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
+    __shared__ __attribute__((aligned(16))) char lds_vbuf[2][kTileBytes];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int H = lane >> 5, r = lane & 31;
+
+    // ---- workgroup -> (head slot, sequence b, row group rg) ------------------------------------
+    const int hslot = blockIdx.x % P.num_q_heads;
+    int b, rg;
+    if (!locate_row_group(P, blockIdx.x / P.num_q_heads, lane, b, rg)) return;
 
     const int seq0 = P.cu_seqlens[b];
     const int L = P.cu_seqlens[b + 1] - seq0;
@@ -195,6 +201,88 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         }
 }
 
+
+// ---- pair-of-heads kernel -----------------------------------------------------------------------
+// Same decomposition in rows, but a wavefront owns its 32 rows for TWO query heads that share a
+// KV head, so that every K / V fragment it fetches from LDS feeds two MFMAs (the one-head form
+// needs 1 KB of LDS reads per MFMA and is bound by that).  512 registers per wavefront, one
+// workgroup per CU; the key loop is the hand-scheduled asm of staircase_pair_core.inc, in which the
+// softmax arithmetic of one tile is issued in the shadow of the next tile's QK MFMAs.  All four
+// wavefronts of a workgroup walk the same number of key tiles; tiles beyond a wavefront's own
+// limit are fully masked.
+#include "staircase_pair_core.inc"
+
+constexpr int kPairLdsBytes = 6 * kTileBytes;     // three K and three V tile slots
+
+// Values the asm reads from scalar registers must be wavefront-uniform in the compiler's eyes.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ const void* uniform(const void* p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const void*)(((uint64_t)hi << 32) | lo);
+}
+
+__global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const StaircaseParams P)
+{
+    extern __shared__ __attribute__((aligned(16))) char lds_pair[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int H = lane >> 5, r = lane & 31;
+
+    const int n_hslots = P.num_q_heads / 2;
+    const int hslot = blockIdx.x % n_hslots;
+    int b, rg;
+    if (!locate_row_group(P, blockIdx.x / n_hslots, lane, b, rg)) return;
+
+    const int seq0 = P.cu_seqlens[b];
+    const int L = P.cu_seqlens[b + 1] - seq0;
+    if (L <= 0) return;
+    const int S = 1 << P.log2_s;
+    const int Lp = ((L + S - 1) >> P.log2_s) << P.log2_s;
+    const int pad = Lp - L;
+    const int row_g0 = rg * kRowsPerWg;
+    if (row_g0 >= Lp) return;
+
+    const int heads_per_kv = P.num_q_heads / P.num_kv_heads;
+    const int kvh = hslot % P.num_kv_heads;                    // launch order: KV head fastest
+    const int head0 = kvh * heads_per_kv + 2 * (hslot / P.num_kv_heads);
+
+    const int row_w0 = row_g0 + wave * 32;
+    const int ip = row_w0 + r;
+    const bool row_ok = ip >= pad && ip < Lp;
+    const int64_t tok = (int64_t)seq0 + (ip - pad);
+    bf16x8 q[2][8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+        load_q(q[h], row_ok ? P.q + tok * P.q_st + (int64_t)(head0 + h) * P.q_sh : nullptr, H);
+
+    auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
+    const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
+
+    const unsigned lds0 = lds_address(lds_pair);
+    const int l16 = lane & 15, gi = (lane >> 4) & 1;
+    PairCoreArgs A;
+    A.ldswr = lds0 + (unsigned)((tid >> 4) * kLdsPitch + (tid & 15) * 16);
+    A.ka = lds0 + (unsigned)(key_of_mfma_row(r) * kLdsPitch + H * 16);
+    A.va = lds0 + (unsigned)(3 * kTileBytes + (4 * (l16 >> 2) + 2 * H) * kLdsPitch + (gi * 16 + (l16 & 3) * 4) * 2);
+    A.jp0 = tid >> 4;
+    A.ck = (unsigned)(tid & 15) * 16u;
+    A.mrel = 2 * H - pad;
+    A.mlim = limit_of(min(ip, Lp - 1)) - pad;
+    A.o0 = P.o + tok * P.o_st + (int64_t)head0 * P.o_sh + 4 * H;
+    A.o1 = A.o0 + P.o_sh;
+    A.ok = row_ok ? 1 : 0;
+    A.kb = uniform((const void*)(P.k + (int64_t)kvh * P.k_sh + ((int64_t)seq0 - pad) * P.k_st));
+    A.vb = uniform((const void*)(P.v + (int64_t)kvh * P.v_sh + ((int64_t)seq0 - pad) * P.v_st));
+    A.krb = (unsigned)uniform((int)(P.k_st * 2));
+    A.vrb = (unsigned)uniform((int)(P.v_st * 2));
+    A.pad = uniform(pad);
+    A.lpm1 = uniform(Lp - 1);
+    A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
+    A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
+    A.c = __int_as_float(uniform(__float_as_int(P.c)));
+    staircase_pair_core(A, q);
+}
+
 }  // namespace
 
 extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
@@ -243,8 +331,19 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence
     const int64_t n_pairs = batch <= 64 ? (total_tokens + (int64_t)batch * (staircase_size + rows_per_wg - 2)) / rows_per_wg
                                         : (int64_t)P.n_row_groups * batch;
-    const int64_t grid = n_pairs * num_q_heads;
+    // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
+    const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
+    const bool pairs = (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
+                       (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31);
+    const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
-    staircase_attn_kernel<<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    if (pairs) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(staircase_pair_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
+        MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
+        staircase_pair_kernel<<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
+    } else {
+        staircase_attn_kernel<<<(unsigned)grid, kThreads, 0, stream>>>(P);
+    }
     return mdx::check_launch("staircase_attn");
 }
