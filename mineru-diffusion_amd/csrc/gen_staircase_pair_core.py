@@ -5,50 +5,58 @@ block-prefill attention kernel for a PAIR of query heads that share a KV head.
 Run  python gen_staircase_pair_core.py > staircase_pair_core.inc  after changing the schedule; the
 .inc file is what the build compiles.
 
-Why assembly: one wavefront per SIMD has to keep the MFMA pipe busy by itself, so LDS fragment reads
-must run several fragments ahead of the MFMA that consumes them and the softmax arithmetic of tile t
-has to be issued in the shadow of the MFMAs of tile t+1.  Both need exact control of instruction
-order and of physical registers that persist across loop iterations, which neither the compiler's
-scheduler nor inline-asm operands (no sub-register access to a 16-register tuple) offer.
+Why assembly: one wavefront per SIMD has to keep the MFMA pipe busy by itself.  Instructions of one
+wavefront issue in order, so LDS fragment reads must run several fragments ahead of the MFMA that
+consumes them and the softmax arithmetic of tile t has to be issued in the shadow of the MFMAs of
+tile t+1.  Both need exact control of instruction order and of physical registers that persist
+across loop iterations, which neither the compiler's scheduler nor inline-asm operands (no
+sub-register access to a 16-register tuple) offer.
 
 Work of one wavefront: 32 query rows x 2 heads, keys in tiles of 64.
-  S^T[key, q] = K . Q^T   A = K fragment (LDS, ds_read_b128), B = Q^T (accumulation registers)
-  O^T[d, q]  += V^T . P^T A = V^T fragment (LDS, two ds_read_b64_tr_b16), B = P^T (registers)
+  S'^T[key, q] = K . (c Q)^T - m    A = K fragment (LDS, ds_read_b128), B = scaled Q^T (accumulation
+                                    registers), C = a tuple holding -m (the stale running max)
+  P = exp2(S'), bf16, in place
+  O^T[d, q]  += V^T . P^T           A = V^T fragment (LDS, two ds_read_b64_tr_b16), B = P^T
 Every K / V^T fragment feeds the MFMAs of both heads.  Register and key maps are those of
-attn_tile.h (key_of_reg, key_of_mfma_row, 272-byte LDS row pitch).
+attn_tile.h (key_of_reg, key_of_mfma_row).
 
-Loop iteration t (S is double-buffered, cb = t & 1):
-  X: 32 MFMAs of QK(t+1) -> S[1-cb]   ||  rescale check(t), softmax(t): S[cb] -> P (in place),
-     tile t+2: staging registers -> LDS, global loads of tile t+3 -> staging registers
-  Y: 32 MFMAs of PV(t)  (P, V slot t) ||  row sums of P(t), row max of S[1-cb], load offsets of tile t+4
-  barrier
-LDS: three slots each for K and V tiles (slot = tile % 3).
+LDS: four slots of 32 KB (tile % 4), K rows then V rows, 256 bytes per row, filled by
+global_load_lds_dwordx4 (1 KB = 4 rows per instruction, 8 instructions per wavefront and tile).  The
+16-byte chunk c of row r sits at position c ^ (r % 16), which makes both fragment read patterns
+bank-conflict free without padding; the XOR shows up as one address register per k-step.
 
-Physical registers (all clobbered; the compiler keeps v0..v39 and a128..a255 for the operands):
-  v40..v63   state and temporaries      v64..v191  S[2][head][sub-tile][16]
-  v192..v223 staging (K, V: 4 x 16 B)   v224..v247 fragment ring (6 x 4)    v248..v255 temporaries
-  a0..a127   O^T[head][d tile][16]      s40..s55   loop state
+Loop iteration t (S is double-buffered, cb = t & 1); the MFMA / fragment stream is continuous:
+  tile t+3: global -> LDS slot (issued early; it has two iterations to land)
+  X: 32 MFMAs of QK(t+1) -> S[1-cb]  ||  rescale check(t), P(t) = exp2(S[cb]) in place
+  Y: 32 MFMAs of PV(t)               ||  row sums of P(t), row max of S[1-cb], addresses of tile t+4
+  wait until tile t+2 has landed, barrier
+
+Physical registers (all clobbered; the compiler keeps v0..v23 and a128..a255 for the operands):
+  v24..v39  K / V^T fragment addresses   v40..v63  state, temporaries, load addresses
+  v64..v191 S[2][head][sub-tile][16]     v192..v223 -m tuples      v224..v247 fragment ring (6 x 4)
+  v248..v255 temporaries                 a0..a127  O^T[head][d tile][16]    s40..s55 loop state
 """
 import sys
 
-PITCH = 272
-TILE_BYTES = 64 * PITCH            # 17408
-V_RING = 3 * TILE_BYTES            # V slots follow the three K slots
+ROW = 256
+K_BYTES = 64 * ROW                 # 16384: K part of a slot; V part follows
+SLOT = 2 * K_BYTES
 RING_DEPTH = 5                     # fragments in flight
-NEG_INF = "v45"                    # holds -inf (a literal would be a second constant-bus read next to vcc)
+DMA_PER_TILE = 8                   # global_load_lds instructions per wavefront and tile
 
 # ---- register names ---------------------------------------------------------------------------
-VPAD, VLPM1, KA, VA, LDSW = "v40", "v41", "v42", "v43", "v44"
-ACC = ["v45", "v46", "v47"]                      # spare temporaries
-OK = [f"v{48 + p}" for p in range(4)]            # global byte offsets of the next K rows to load
-OV = [f"v{52 + p}" for p in range(4)]
-M = ["v56", "v57"]
-L = ["v58", "v59"]
-MX = ["v60", "v61"]
-MREL, JP = "v62", "v63"
+KA = [f"v{24 + i}" for i in range(8)]            # K fragment address of k-step ks (current slot)
+VA = [[f"v{32 + 4 * q + dt}" for dt in range(4)] for q in range(2)]   # V^T address [lo / hi][d tile]
+VPAD, VLPM1, JPL, NEG_INF = "v40", "v41", "v42", "v43"
+L = ["v46", "v47"]
+MX = ["v48", "v49"]
+MREL = "v50"
+GK = [f"v{56 + i}" for i in range(4)]            # global byte offsets of the rows the next loads fetch
+GV = [f"v{60 + i}" for i in range(4)]
 T = [f"v{248 + i}" for i in range(8)]
-S_T, S_KEY0, S_R0, S_R1, S_R2, S_TMP = "s40", "s41", "s42", "s43", "s44", "s45"
-S_SAVE = "s[46:47]"
+S_T, S_KEY0, S_R0, S_R1, S_R2, S_R3, S_TMP = "s40", "s41", "s42", "s43", "s44", "s45", "s46"
+S_SAVE = "s[48:49]"
+S_DST = "s50"
 
 
 def sreg(b, h, u, i):
@@ -65,6 +73,11 @@ def ptup(b, h, u, t):
     return f"v[{r}:{r + 3}]"
 
 
+def negm(h, i=None):
+    r = 192 + 16 * h
+    return f"v[{r}:{r + 15}]" if i is None else f"v{r + i}"
+
+
 def otup(h, dt):
     r = 64 * h + 16 * dt
     return f"a[{r}:{r + 15}]"
@@ -75,42 +88,17 @@ def ring(i):
     return f"v[{r}:{r + 3}]", f"v[{r}:{r + 1}]", f"v[{r + 2}:{r + 3}]"
 
 
-def stg(kv, p):
-    r = 192 + 16 * kv + 4 * p
-    return f"v[{r}:{r + 3}]"
-
-
-class Lds:
-    """Tracks LDS operations in flight so that waits can be written as exact lgkmcnt values."""
-
-    def __init__(self):
-        self.issued = 0
-
-    def op(self, out, text):
-        out.append(text)
-        self.issued += 1
-        return self.issued - 1
-
-    def wait(self, out, idx):
-        n = self.issued - 1 - idx
-        assert 0 <= n <= 15, n
-        out.append(f"s_waitcnt lgkmcnt({n})")
-
-    def drain(self, out):
-        out.append("s_waitcnt lgkmcnt(0)")
-        self.issued = 0
-
-
 # ---- VALU fragments -----------------------------------------------------------------------------
 def key_const(u, i):
     return 32 * u + 16 * (i >> 3) + 4 * (i & 3) + ((i >> 2) & 1)
 
 
 def softmax_ops(cb, masked):
-    """S[cb] -> P in place, both heads.  Chunks of 8 values; the conversion of a chunk is issued
-    one chunk after its exponentials (v_exp results need a gap before a non-transcendental use)."""
+    """S[cb] -> P in place, both heads, in the order PV consumes it.  Chunks of 8 values; the
+    conversion of a chunk is issued one chunk after its exponentials (a v_exp result needs a gap
+    before a non-transcendental instruction reads it)."""
     ops = []
-    chunks = [(h, u, t) for u in range(2) for t in range(2) for h in range(2)]   # PV consumes (u, t) in this order
+    chunks = [(h, u, t) for u in range(2) for t in range(2) for h in range(2)]
     pending = None
     for (h, u, t) in chunks:
         regs = [sreg(cb, h, u, 8 * t + j) for j in range(8)]
@@ -119,8 +107,6 @@ def softmax_ops(cb, masked):
                 ops.append(f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}")
                 ops.append(f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]")
                 ops.append(f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc")
-        for r in regs:
-            ops.append(f"v_fma_f32 v{r}, v{r}, %[c], -{M[h]}")
         for r in regs:
             ops.append(f"v_exp_f32_e32 v{r}, v{r}")
         if pending:
@@ -154,77 +140,88 @@ def rowsum_ops(cb):
 
 
 def rowmax_ops(b):
-    """MX[h] = max over this query's 64 keys of S[b][h] (raw scores, both half-waves)."""
+    """MX[h] = max over this query's 64 keys of S[b][h] (both half-waves); the two heads' chains
+    alternate so that no instruction depends on its predecessor."""
     ops = []
+    regs = {h: [sreg(b, h, u, i) for u in range(2) for i in range(16)] for h in range(2)}
+    acc = {h: (T[2 * h], T[2 * h + 1]) for h in range(2)}
     for h in range(2):
-        regs = [sreg(b, h, u, i) for u in range(2) for i in range(16)]
-        a, c = T[2 * h], T[2 * h + 1]
-        ops.append(f"v_max3_f32 {a}, v{regs[0]}, v{regs[1]}, v{regs[2]}")
-        ops.append(f"v_max3_f32 {c}, v{regs[3]}, v{regs[4]}, v{regs[5]}")
-        rest = regs[6:]                              # 26 values, two per further step, alternating chains
-        for i in range(0, len(rest), 2):
-            d = a if (i >> 1) % 2 == 0 else c
-            ops.append(f"v_max3_f32 {d}, {d}, v{rest[i]}, v{rest[i + 1]}")
-        ops.append(f"v_max_f32_e32 {a}, {a}, {c}")
+        ops.append(f"v_max3_f32 {acc[h][0]}, v{regs[h][0]}, v{regs[h][1]}, v{regs[h][2]}")
     for h in range(2):
-        a, c = T[2 * h], T[2 * h + 1]
-        ops.append(f"v_mov_b32_e32 {c}, {a}")
+        ops.append(f"v_max3_f32 {acc[h][1]}, v{regs[h][3]}, v{regs[h][4]}, v{regs[h][5]}")
+    for i in range(6, 32, 2):
+        for h in range(2):
+            d = acc[h][(i >> 1) & 1]
+            ops.append(f"v_max3_f32 {d}, {d}, v{regs[h][i]}, v{regs[h][i + 1]}")
+    for h in range(2):
+        ops.append(f"v_max_f32_e32 {acc[h][0]}, {acc[h][0]}, {acc[h][1]}")
+    for h in range(2):
+        ops.append(f"v_mov_b32_e32 {acc[h][1]}, {acc[h][0]}")
     ops.append("s_nop 1")
     for h in range(2):
-        a, c = T[2 * h], T[2 * h + 1]
-        ops.append(f"v_permlane32_swap_b32_e32 {a}, {c}")
+        ops.append(f"v_permlane32_swap_b32_e32 {acc[h][0]}, {acc[h][1]}")
     ops.append("s_nop 1")
     for h in range(2):
-        a, c = T[2 * h], T[2 * h + 1]
-        ops.append(f"v_max_f32_e32 {MX[h]}, {a}, {c}")
+        ops.append(f"v_max_f32_e32 {MX[h]}, {acc[h][0]}, {acc[h][1]}")
     return ops
 
 
 def load_offset_ops():
-    """Byte offsets of the rows the next global loads fetch (rows clamped into the sequence), then JP += 64."""
+    """Byte offsets of the rows the next global loads fetch (rows clamped into the sequence), then JPL += 64."""
     ops = []
-    for p in range(4):
-        ops.append(f"v_add_u32_e32 {T[6]}, {16 * p}, {JP}")
+    for i in range(4):
+        ops.append(f"v_add_u32_e32 {T[6]}, {16 * i}, {JPL}")
         ops.append(f"v_med3_i32 {T[6]}, {T[6]}, {VPAD}, {VLPM1}")
-        ops.append(f"v_mul_lo_u32 {OK[p]}, {T[6]}, %[krb]")
-        ops.append(f"v_mul_lo_u32 {OV[p]}, {T[6]}, %[vrb]")
-        ops.append(f"v_add_u32_e32 {OK[p]}, {OK[p]}, %[ck]")
-        ops.append(f"v_add_u32_e32 {OV[p]}, {OV[p]}, %[ck]")
-    ops.append(f"v_add_u32_e32 {JP}, 64, {JP}")
+        ops.append(f"v_mad_u32_u24 {GK[i]}, {T[6]}, %[krb], %[ch]")
+        ops.append(f"v_mad_u32_u24 {GV[i]}, {T[6]}, %[vrb], %[ch]")
+    ops.append(f"v_add_u32_e32 {JPL}, 64, {JPL}")
     return ops
 
 
-def global_loads():
-    out = []
-    for p in range(4):
-        out.append(f"global_load_dwordx4 {stg(0, p)}, {OK[p]}, %[kb]")
-        out.append(f"global_load_dwordx4 {stg(1, p)}, {OV[p]}, %[vb]")
-    return out
+def dma_ops(slot_sreg):
+    """The 8 global -> LDS loads of one tile into the slot whose byte offset is in slot_sreg; each
+    entry is the instruction group of one load (M0 = LDS destination of lane 0)."""
+    groups = []
+    for i in range(4):
+        for kv, (off, base) in enumerate(((GK, "%[kb]"), (GV, "%[vb]"))):
+            g = [f"s_add_u32 m0, {S_DST}, {4096 * i + K_BYTES * kv}", "s_nop 0",
+                 f"global_load_lds_dwordx4 {off[i]}, {base}"]
+            if i == 0 and kv == 0:
+                g = [f"s_add_u32 {S_DST}, {slot_sreg}, %[wrow]"] + g
+            groups.append(g)
+    return groups
 
 
-def stage_writes(lds, out, slot_sreg):
-    """Staging registers -> LDS slot whose byte offset is in slot_sreg."""
-    out.append("s_waitcnt vmcnt(0)")
-    out.append(f"v_add_u32_e32 {LDSW}, {slot_sreg}, %[ldswr]")
-    for p in range(4):
-        lds.op(out, f"ds_write_b128 {LDSW}, {stg(0, p)} offset:{4352 * p}")
-        lds.op(out, f"ds_write_b128 {LDSW}, {stg(1, p)} offset:{V_RING + 4352 * p}")
+def address_ops():
+    """Fragment addresses of this iteration: K of slot R1 (tile t+1), V of slot R0 (tile t)."""
+    ops = [f"v_add_u32_e32 {KA[0]}, {S_R1}, %[ka]"]
+    for ks in range(1, 8):
+        ops.append(f"v_xor_b32_e32 {KA[ks]}, {hex(ks << 5)}, {KA[0]}")
+    for q, name in enumerate(("%[val]", "%[vah]")):
+        ops.append(f"v_add_u32_e32 {VA[q][0]}, {S_R0}, {name}")
+        for dt in range(1, 4):
+            ops.append(f"v_xor_b32_e32 {VA[q][dt]}, {hex(dt << 6)}, {VA[q][0]}")
+    return ops
 
 
-def check_rescale(uid):
-    """Running-max update of both heads from MX (lazy: only when some query exceeds the stale max
-    by more than 2^8); the rare path rescales l and O^T (accumulation registers) in place."""
+def check_rescale(uid, cb):
+    """Lazy running-max update from MX = row max of S' = c s - m: only when some query exceeds the
+    stale max by more than 2^8.  The rare path moves m up by delta = max(MX, 0): the -m tuple and
+    the scores of tile t (computed with the old m) go down by delta, l and O^T (accumulation
+    registers) are scaled by 2^-delta."""
     out = []
     for h in range(2):
         lab = f".Lskip_{uid}_{h}_%="
-        out.append(f"v_mul_f32_e32 {T[0]}, %[c], {MX[h]}")
-        out.append(f"v_max_f32_e32 {T[0]}, {T[0]}, {M[h]}")
-        out.append(f"v_add_f32_e32 {T[1]}, 0x41000000, {M[h]}")
-        out.append(f"v_cmp_gt_f32_e32 vcc, {T[0]}, {T[1]}")
+        out.append(f"v_cmp_lt_f32_e32 vcc, 0x41000000, {MX[h]}")
         out.append(f"s_cbranch_vccz {lab}")
-        out.append(f"v_sub_f32_e32 {T[1]}, {M[h]}, {T[0]}")
-        out.append(f"v_exp_f32_e32 {T[1]}, {T[1]}")
-        out.append(f"v_mov_b32_e32 {M[h]}, {T[0]}")
+        out.append(f"v_max_f32_e32 {T[0]}, 0, {MX[h]}")
+        out.append(f"v_exp_f32_e64 {T[1]}, -{T[0]}")
+        for i in range(16):
+            out.append(f"v_sub_f32_e32 {negm(h, i)}, {negm(h, i)}, {T[0]}")
+        for u in range(2):
+            for i in range(16):
+                r = sreg(cb, h, u, i)
+                out.append(f"v_sub_f32_e32 v{r}, v{r}, {T[0]}")
         out.append("s_nop 15")                      # the MFMAs of the previous tile's PV have long finished; margin only
         out.append(f"v_mul_f32_e32 {L[h]}, {L[h]}, {T[1]}")
         for i in range(64):
@@ -238,122 +235,136 @@ def check_rescale(uid):
     return out
 
 
-# ---- MFMA streams -------------------------------------------------------------------------------
-def qk_stream(nb):
-    """[(reads, mfmas)] per K fragment n: fragment (u = n & 1, ks = n >> 1) -> S[nb][h][u] for h = 0, 1."""
+# ---- MFMA / fragment stream ----------------------------------------------------------------------
+def qk_items(nb):
+    """K fragment n = (u = n & 1, ks = n >> 1) -> S[nb][h][u] for h = 0, 1."""
     items = []
     for n in range(16):
         u, ks = n & 1, n >> 1
-        frag = ring(n)[0]
-        rd = [f"ds_read_b128 {frag}, {KA} offset:{u * 32 * PITCH + ks * 32}"]
-        mf = []
-        for h in range(2):
-            c = "0" if ks == 0 else stup(nb, h, u)
-            mf.append(f"v_mfma_f32_32x32x16_bf16 {stup(nb, h, u)}, {frag}, %[q{h}{ks}], {c}")
+        rd = lambda frag, u=u, ks=ks: [f"ds_read_b128 {frag[0]}, {KA[ks]}" + (f" offset:{u * 32 * ROW}" if u else "")]
+        mf = lambda frag, u=u, ks=ks: [
+            f"v_mfma_f32_32x32x16_bf16 {stup(nb, h, u)}, {frag[0]}, %[q{h}{ks}], {negm(h) if ks == 0 else stup(nb, h, u)}"
+            for h in range(2)]
         items.append((rd, mf))
     return items
 
 
-def pv_stream(cb):
-    """Fragment m: (u, t, dt) = (m >> 3, (m >> 2) & 1, m & 3); O^T[h][dt] += V^T frag . P[h][u][t]."""
+def pv_items(cb):
+    """V^T fragment m = (u, t, dt) = (m >> 3, (m >> 2) & 1, m & 3); O^T[h][dt] += fragment . P[h][u][t]."""
     items = []
     for m in range(16):
         u, t, dt = m >> 3, (m >> 2) & 1, m & 3
-        frag, lo, hi = ring(m)
-        o = (u * 32 + t * 16) * PITCH + dt * 64
-        rd = [f"ds_read_b64_tr_b16 {lo}, {VA} offset:{o}", f"ds_read_b64_tr_b16 {hi}, {VA} offset:{o + PITCH}"]
-        mf = [f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)]
+        o = (u * 32 + t * 16) * ROW
+        sfx = f" offset:{o}" if o else ""
+        rd = lambda frag, dt=dt, sfx=sfx: [f"ds_read_b64_tr_b16 {frag[1]}, {VA[0][dt]}{sfx}",
+                                           f"ds_read_b64_tr_b16 {frag[2]}, {VA[1][dt]}{sfx}"]
+        mf = lambda frag, u=u, t=t, dt=dt: [
+            f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)]
         items.append((rd, mf))
     return items
 
 
-def interleave(out, lds, items, valu, extras=None):
-    """MFMA stream with a read-ahead of RING_DEPTH fragments; VALU ops are dealt evenly into the
-    slots after each MFMA; extras = {fragment index: [instructions or callables]} are placed after
-    that fragment's MFMAs."""
+def stream(out, items, valu_plan, extras=None, head=None, c0_zero=False):
+    """Emits the fragment reads RING_DEPTH items ahead of the MFMAs that consume them.
+    valu_plan: list of (first MFMA slot, last MFMA slot + 1, ops): ops are dealt evenly into the
+    slots (one slot follows each MFMA).  extras: {item index: [instruction groups]} placed after
+    that item's MFMAs.  head: instructions issued right after the first reads (they run while the
+    reads are in flight).  Waits are exact lgkmcnt values: LDS operations complete in order."""
     extras = extras or {}
     n_slots = 2 * len(items)
-    per = [len(valu) // n_slots + (1 if i < len(valu) % n_slots else 0) for i in range(n_slots)]
-    vi = 0
-    ids = {}
+    per_slot = [[] for _ in range(n_slots)]
+    for (a, b, ops) in valu_plan:
+        n = b - a
+        base, rem = divmod(len(ops), n)
+        k = 0
+        for i in range(n):
+            c = base + (1 if i < rem else 0)
+            per_slot[a + i] += ops[k:k + c]
+            k += c
+    issued = 0
+    last_id = {}
+
+    def issue_reads(n):
+        nonlocal issued
+        for r in items[n][0](ring(n)):
+            out.append(r)
+            issued += 1
+        last_id[n] = issued - 1
+
     for n in range(min(RING_DEPTH, len(items))):
-        for r in items[n][0]:
-            ids[n] = lds.op(out, r)
+        issue_reads(n)
+    if head:
+        out.extend(head)
     slot = 0
     for n, (rd, mf) in enumerate(items):
-        lds.wait(out, ids[n])
-        for mi, mfma in enumerate(mf):
+        w = issued - 1 - last_id[n]
+        assert 0 <= w <= 15
+        out.append(f"s_waitcnt lgkmcnt({w})")
+        for mfma in mf(ring(n)):
+            if c0_zero:
+                mfma = mfma.replace(f", {negm(0)}", ", 0").replace(f", {negm(1)}", ", 0")
             out.append(mfma)
-            for _ in range(per[slot]):
-                out.append(valu[vi])
-                vi += 1
+            out.extend(per_slot[slot])
             slot += 1
-        nxt = n + RING_DEPTH
-        if nxt < len(items):
-            for r in items[nxt][0]:
-                ids[nxt] = lds.op(out, r)
-        for e in extras.get(n, []):
-            if callable(e):
-                e(out)
-            else:
-                out.append(e)
-    assert vi == len(valu)
+        if n + RING_DEPTH < len(items):
+            issue_reads(n + RING_DEPTH)
+        for g in extras.get(n, []):
+            out.extend(g)
 
 
 # ---- program ------------------------------------------------------------------------------------
 def prologue():
     out = []
-    lds = Lds()
     out += [f"v_mov_b32_e32 {NEG_INF}, 0xff800000", f"v_mov_b32_e32 {VPAD}, %[pad]", f"v_mov_b32_e32 {VLPM1}, %[lpm1]",
-            f"v_mov_b32_e32 {MREL}, %[mrel]", f"v_mov_b32_e32 {JP}, %[jp0]"]
+            f"v_mov_b32_e32 {MREL}, %[mrel]", f"v_mov_b32_e32 {JPL}, %[jpl]"]
     for h in range(2):
-        out += [f"v_mov_b32_e32 {M[h]}, 0xf149f2ca", f"v_mov_b32_e32 {L[h]}, 0"]      # -1e30
+        out.append(f"v_mov_b32_e32 {L[h]}, 0")
     for i in range(128):
         out.append(f"v_accvgpr_write_b32 a{i}, 0")
-    out += [f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_KEY0}, 0", f"s_mov_b32 {S_R0}, 0",
-            f"s_mov_b32 {S_R1}, {TILE_BYTES}", f"s_mov_b32 {S_R2}, {2 * TILE_BYTES}"]
-    # tiles 0 and 1 -> LDS slots 0 and 1; tile 2 -> staging registers; offsets of tile 3 prepared
-    for slot in (S_R0, S_R1):
+    out += [f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_KEY0}, 0", f"s_mov_b32 {S_R0}, 0", f"s_mov_b32 {S_R1}, {SLOT}",
+            f"s_mov_b32 {S_R2}, {2 * SLOT}", f"s_mov_b32 {S_R3}, {3 * SLOT}"]
+    # tiles 0, 1, 2 -> slots 0, 1, 2; addresses of tile 3 prepared
+    for slot in (S_R0, S_R1, S_R2):
         out += load_offset_ops()
-        out += global_loads()
-        stage_writes(lds, out, slot)
+        for g in dma_ops(slot):
+            out += g
     out += load_offset_ops()
-    out += global_loads()
-    out += load_offset_ops()
-    lds.drain(out)
-    out.append("s_barrier")
-    # QK(0) -> S[0], row max of tile 0
-    out.append(f"v_add_u32_e32 {KA}, {S_R0}, %[ka]")
-    interleave(out, lds, qk_stream(0), [])
+    out += [f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]          # tiles 0 and 1 have landed
+    # QK(0) with C = 0, then m = row max of tile 0: -m tuples and S[0] -= m
+    out.append(f"v_add_u32_e32 {KA[0]}, {S_R0}, %[ka]")
+    for ks in range(1, 8):
+        out.append(f"v_xor_b32_e32 {KA[ks]}, {hex(ks << 5)}, {KA[0]}")
+    stream(out, qk_items(0), [], c0_zero=True)
     out.append("s_nop 15")
     out += rowmax_ops(0)
+    for h in range(2):
+        for i in range(16):
+            out.append(f"v_sub_f32_e32 {negm(h, i)}, 0, {MX[h]}")
+        for u in range(2):
+            for i in range(16):
+                r = sreg(0, h, u, i)
+                out.append(f"v_sub_f32_e32 v{r}, v{r}, {MX[h]}")
+        out.append(f"v_mov_b32_e32 {MX[h]}, 0")
     return out
 
 
 def body(cb, masked):
     uid = f"{cb}{int(masked)}"
     out = []
-    lds = Lds()
     nb = 1 - cb
-    out += check_rescale(uid)
-    # ---- X
-    out.append(f"v_add_u32_e32 {KA}, {S_R1}, %[ka]")
-    extras = {1: [lambda o: stage_writes(lds, o, S_R2)], 7: global_loads()}
-    interleave(out, lds, qk_stream(nb), softmax_ops(cb, masked), extras)
-    out.append("s_nop 1")
-    # ---- Y
-    out.append(f"v_add_u32_e32 {VA}, {S_R0}, %[va]")
-    yv = rowsum_ops(cb)
-    pre = ["s_nop 7"]                       # S[nb] was written by the last MFMAs of X
-    yv_late = rowmax_ops(nb) + load_offset_ops()
-    items = pv_stream(cb)
-    # row max may only start once the QK MFMAs have retired: give the sums the first slots
-    interleave(out, lds, items, yv + pre + yv_late)
-    lds.drain(out)
-    # ---- loop state
-    out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_TMP}",
+    sm = softmax_ops(cb, masked)
+    yv = rowsum_ops(cb) + ["s_nop 7"] + rowmax_ops(nb) + load_offset_ops()
+    items = qk_items(nb) + pv_items(cb)
+    dma = dma_ops(S_R3)
+    extras = {1 + i: [dma[i]] for i in range(DMA_PER_TILE)}
+    out += address_ops()
+    # P(h, u, t) is first read by PV item 4 (2u + t): the softmax may run 8 slots into the PV part
+    stream(out, items, [(0, 40, sm), (40, 64, yv)], extras, head=check_rescale(uid, cb))
+    # ---- loop state; tile t+2 (issued one iteration ago) must have landed before the barrier
+    out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_R3}",
+            f"s_mov_b32 {S_R3}, {S_TMP}",
             f"s_add_i32 {S_T}, {S_T}, 1", f"s_add_i32 {S_KEY0}, {S_KEY0}, 64", f"v_add_u32_e32 {MREL}, 64, {MREL}",
-            "s_barrier"]
+            f"s_waitcnt vmcnt({DMA_PER_TILE}) lgkmcnt(0)", "s_barrier"]
     return out
 
 
@@ -405,20 +416,21 @@ def program():
 HEADER = '''// GENERATED by gen_staircase_pair_core.py -- do not edit; change the generator and regenerate.
 //
 // Key loop of the staircase attention kernel for a pair of query heads (see the generator's
-// docstring for the schedule and the register map).  Everything between the loads of Q and the
-// stores of O happens inside this one asm statement; the physical registers it uses are declared
-// as clobbers, the operands are read-only.
+// docstring for the schedule, the LDS layout and the register map).  Everything between the loads
+// of Q and the stores of O happens inside this one asm statement; the physical registers it uses
+// are declared as clobbers, the operands are read-only.
 struct PairCoreArgs {
-    unsigned ldswr, ka, va;          // per-lane LDS byte addresses: staging write, K fragment read, V^T fragment read (slot 0)
-    int jp0;                         // row of the tile this thread stages (threadIdx / 16)
-    unsigned ck;                     // byte offset of this thread's 16-byte chunk inside a row
+    unsigned ka;                     // per-lane LDS byte address of this lane's K fragment of k-step 0 in slot 0
+    unsigned val, vah;               // same for the two rows of the V^T fragment of d tile 0
+    int jpl;                         // row of the tile whose chunk this lane loads (first of four, 16 apart)
+    unsigned ch;                     // byte offset inside a K / V row of the 16-byte chunk this lane loads
     int mrel, mlim;                  // key mask: key visible iff unsigned(key0 + const + mrel) < mlim
     __bf16* o0; __bf16* o1;          // output rows of the two heads (+ 4 * half-wave elements)
     int ok;                          // this lane's query row exists
     const void* kb; const void* vb;  // K / V of this KV head, at the (virtual) row of padded key 0
     unsigned krb, vrb;               // bytes between consecutive K / V rows
+    unsigned wrow;                   // LDS byte address of the first row this wavefront loads in slot 0
     int pad, lpm1, nt, whm;          // first valid padded key, last valid padded key, key tiles, first limit of this wavefront
-    float c;                         // softmax scale * log2(e)
 };
 
 __device__ __forceinline__ void staircase_pair_core(const PairCoreArgs& A, const bf16x8 (&q)[2][8])
@@ -431,17 +443,17 @@ def main():
     prog = program()
     text = "\n".join(f'        "{line}\\n"' for line in prog)
     qops = ", ".join(f'[q{h}{ks}] "a"(q[{h}][{ks}])' for h in range(2) for ks in range(8))
-    vclob = ", ".join(f'"v{r}"' for r in range(40, 256))
+    vclob = ", ".join(f'"v{r}"' for r in range(24, 256))
     aclob = ", ".join(f'"a{r}"' for r in range(0, 128))
     sclob = ", ".join(f'"s{r}"' for r in range(40, 56))
     tail = f'''
         :
-        : [ldswr] "v"(A.ldswr), [ka] "v"(A.ka), [va] "v"(A.va), [jp0] "v"(A.jp0), [ck] "v"(A.ck),
+        : [ka] "v"(A.ka), [val] "v"(A.val), [vah] "v"(A.vah), [jpl] "v"(A.jpl), [ch] "v"(A.ch),
           [mrel] "v"(A.mrel), [mlim] "v"(A.mlim), [o0] "v"(A.o0), [o1] "v"(A.o1), [ok] "v"(A.ok),
-          [kb] "s"(A.kb), [vb] "s"(A.vb), [krb] "s"(A.krb), [vrb] "s"(A.vrb), [pad] "s"(A.pad), [lpm1] "s"(A.lpm1),
-          [nt] "s"(A.nt), [whm] "s"(A.whm), [c] "s"(A.c), [ones] "s"(0x3f803f80u),
+          [kb] "s"(A.kb), [vb] "s"(A.vb), [krb] "s"(A.krb), [vrb] "s"(A.vrb), [wrow] "s"(A.wrow),
+          [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm), [ones] "s"(0x3f803f80u),
           {qops}
-        : "memory", "vcc", "scc", {sclob},
+        : "memory", "vcc", "scc", "m0", {sclob},
           {vclob},
           {aclob});
 }}

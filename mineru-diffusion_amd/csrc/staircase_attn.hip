@@ -212,7 +212,8 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 // limit are fully masked.
 #include "staircase_pair_core.inc"
 
-constexpr int kPairLdsBytes = 6 * kTileBytes;     // three K and three V tile slots
+constexpr int kPairSlots = 4;                     // LDS slots of one K tile + one V tile, 256-byte rows
+constexpr int kPairLdsBytes = kPairSlots * 2 * kTileKeys * kRowBytes;
 
 // Values the asm reads from scalar registers must be wavefront-uniform in the compiler's eyes.
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
@@ -224,7 +225,7 @@ __device__ __forceinline__ const void* uniform(const void* p) {
 
 __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const StaircaseParams P)
 {
-    extern __shared__ __attribute__((aligned(16))) char lds_pair[];
+    extern __shared__ __attribute__((aligned(1024))) char lds_pair[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
 
@@ -250,10 +251,16 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     const int ip = row_w0 + r;
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
+    // Q^T fragments, pre-multiplied by scale * log2(e) (the MFMA then yields scores in log2 units)
     bf16x8 q[2][8];
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < 2; ++h) {
         load_q(q[h], row_ok ? P.q + tok * P.q_st + (int64_t)(head0 + h) * P.q_sh : nullptr, H);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) q[h][ks][j] = (__bf16)((float)q[h][ks][j] * P.c);
+    }
 
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
     const int wg_hi = limit_of(min(row_g0 + kRowsPerWg - 1, Lp - 1));
@@ -261,11 +268,19 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     const unsigned lds0 = lds_address(lds_pair);
     const int l16 = lane & 15, gi = (lane >> 4) & 1;
     PairCoreArgs A;
-    A.ldswr = lds0 + (unsigned)((tid >> 4) * kLdsPitch + (tid & 15) * 16);
-    A.ka = lds0 + (unsigned)(key_of_mfma_row(r) * kLdsPitch + H * 16);
-    A.va = lds0 + (unsigned)(3 * kTileBytes + (4 * (l16 >> 2) + 2 * H) * kLdsPitch + (gi * 16 + (l16 & 3) * 4) * 2);
-    A.jp0 = tid >> 4;
-    A.ck = (unsigned)(tid & 15) * 16u;
+    {   // K fragment of k-step 0: row key_of_mfma_row(r), chunk H, swizzled by row % 16
+        const int row = key_of_mfma_row(r), f = row & 15;
+        A.ka = lds0 + (unsigned)(row * kRowBytes + ((f & 14) << 4) + (((H ^ f) & 1) << 4));
+    }
+    {   // V^T fragment of d tile 0: rows rho, rho + 1; chunk c0, 8-byte half sub
+        const int rho = 4 * (l16 >> 2) + 2 * H, c0 = gi * 2 + ((l16 & 3) >> 1), sub = (l16 & 1) * 8;
+        const unsigned vbase = lds0 + (unsigned)(kTileKeys * kRowBytes);
+        A.val = vbase + (unsigned)(rho * kRowBytes + (((rho & 12) | (c0 ^ (rho & 3))) << 4) + sub);
+        A.vah = vbase + (unsigned)((rho + 1) * kRowBytes + (((rho & 12) | (c0 ^ ((rho & 3) | 1))) << 4) + sub);
+    }
+    A.jpl = 4 * wave + (lane >> 4);
+    A.ch = (unsigned)(((lane & 15) ^ (A.jpl & 15)) * 16);
+    A.wrow = (unsigned)uniform((int)(lds0 + (unsigned)(4 * wave * kRowBytes)));
     A.mrel = 2 * H - pad;
     A.mlim = limit_of(min(ip, Lp - 1)) - pad;
     A.o0 = P.o + tok * P.o_st + (int64_t)head0 * P.o_sh + 4 * H;
@@ -279,7 +294,6 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.lpm1 = uniform(Lp - 1);
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
-    A.c = __int_as_float(uniform(__float_as_int(P.c)));
     staircase_pair_core(A, q);
 }
 
@@ -334,7 +348,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
     const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
     const bool pairs = (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
-                       (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31);
+                       (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
     if (pairs) {
