@@ -28,13 +28,15 @@ bank-conflict free without padding; the XOR shows up as one address register per
 Loop iteration t (S is double-buffered, cb = t & 1); the MFMA / fragment stream is continuous:
   tile t+3: global -> LDS slot (issued early; it has two iterations to land)
   X: 32 MFMAs of QK(t+1) -> S[1-cb]  ||  rescale check(t), P(t) = exp2(S[cb]) in place
-  Y: 32 MFMAs of PV(t)               ||  row sums of P(t), row max of S[1-cb], addresses of tile t+4
+  Y: 32 MFMAs of PV(t) + 8 of ones . P^T (row sums)  ||  row max of S[1-cb], addresses of tile t+4,
+     loads of tile t+3
   wait until tile t+2 has landed, barrier
 
 Physical registers (all clobbered; the compiler keeps v0..v23 and a128..a255 for the operands):
   v24..v39  K / V^T fragment addresses   v40..v63  state, temporaries, load addresses
   v64..v191 S[2][head][sub-tile][16]     v192..v223 -m tuples      v224..v247 fragment ring (6 x 4)
-  v248..v255 temporaries                 a0..a127  O^T[head][d tile][16]    s40..s55 loop state
+  v248..v255 temporaries                 a0..a127  O^T[head][d tile][16]    a192..a223 row sums
+  s40..s55 loop state
 """
 import sys
 
@@ -48,7 +50,7 @@ DMA_PER_TILE = 8                   # global_load_lds instructions per wavefront 
 KA = [f"v{24 + i}" for i in range(8)]            # K fragment address of k-step ks (current slot)
 VA = [[f"v{32 + 4 * q + dt}" for dt in range(4)] for q in range(2)]   # V^T address [lo / hi][d tile]
 VPAD, VLPM1, JPL, NEG_INF = "v40", "v41", "v42", "v43"
-L = ["v46", "v47"]
+ONES = "v[52:55]"                                # A fragment of bf16 ones: an MFMA with it sums the rows of P^T
 MX = ["v48", "v49"]
 MREL = "v50"
 GK = [f"v{56 + i}" for i in range(4)]            # global byte offsets of the rows the next loads fetch
@@ -83,6 +85,12 @@ def otup(h, dt):
     return f"a[{r}:{r + 15}]"
 
 
+def lacc(h, i=None):
+    """Row sums l of head h: every register of the tuple holds the sum of its lane's query."""
+    r = 192 + 16 * h
+    return f"a[{r}:{r + 15}]" if i is None else f"a{r + i}"
+
+
 def ring(i):
     r = 224 + 4 * (i % 6)
     return f"v[{r}:{r + 3}]", f"v[{r}:{r + 1}]", f"v[{r + 2}:{r + 3}]"
@@ -94,9 +102,11 @@ def key_const(u, i):
 
 
 def softmax_ops(cb, masked):
-    """S[cb] -> P in place, both heads, in the order PV consumes it.  Chunks of 8 values; the
-    conversion of a chunk is issued one chunk after its exponentials (a v_exp result needs a gap
-    before a non-transcendental instruction reads it)."""
+    """S[cb] -> P in place, both heads, in the order PV consumes it.  Chunks of 8 values; the row
+    sums and the conversion of a chunk are issued one chunk after its exponentials (a v_exp result
+    needs a gap before a non-transcendental instruction reads it).  The row sums are not computed
+    here: the PV part multiplies P^T by a fragment of ones (8 MFMAs per tile instead of 64 adds;
+    the wavefront is bound by instruction issue, not by the matrix pipe)."""
     ops = []
     chunks = [(h, u, t) for u in range(2) for t in range(2) for h in range(2)]
     pending = None
@@ -115,27 +125,6 @@ def softmax_ops(cb, masked):
         pending = [f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}" for j in range(4)]
     ops.append("s_nop 0")
     ops += pending
-    return ops
-
-
-def rowsum_ops(cb):
-    """l[h] += sum of the bf16 probabilities of tile t (two accumulation chains per head)."""
-    ops = []
-    part = {0: (L[0], T[4]), 1: (L[1], T[5])}
-    ops.append(f"v_mov_b32_e32 {T[4]}, 0")
-    ops.append(f"v_mov_b32_e32 {T[5]}, 0")
-    k = 0
-    for u in range(2):
-        for t in range(2):
-            for j in range(4):
-                for h in range(2):
-                    r = sreg(cb, h, u, 8 * t + j)
-                    acc = part[h][k & 1]
-                    ops.append(f"v_dot2_f32_bf16 {acc}, v{r}, %[ones], {acc}")
-                k += 1
-    ops.append("s_nop 3")        # a dot result needs 3 wait states before a VALU of another kind reads it
-    for h in range(2):
-        ops.append(f"v_add_f32_e32 {L[h]}, {L[h]}, {part[h][1]}")
     return ops
 
 
@@ -179,16 +168,15 @@ def load_offset_ops():
 
 
 def dma_ops(slot_sreg):
-    """The 8 global -> LDS loads of one tile into the slot whose byte offset is in slot_sreg; each
-    entry is the instruction group of one load (M0 = LDS destination of lane 0)."""
+    """The 8 global -> LDS loads of one tile into the slot whose byte offset is in slot_sreg, as
+    (M0 write, load) pairs: M0 = LDS destination of lane 0; other instructions must separate the two."""
     groups = []
     for i in range(4):
         for kv, (off, base) in enumerate(((GK, "%[kb]"), (GV, "%[vb]"))):
-            g = [f"s_add_u32 m0, {S_DST}, {4096 * i + K_BYTES * kv}", "s_nop 0",
-                 f"global_load_lds_dwordx4 {off[i]}, {base}"]
+            first = [f"s_add_u32 m0, {S_DST}, {4096 * i + K_BYTES * kv}"]
             if i == 0 and kv == 0:
-                g = [f"s_add_u32 {S_DST}, {slot_sreg}, %[wrow]"] + g
-            groups.append(g)
+                first = [f"s_add_u32 {S_DST}, {slot_sreg}, %[wrow]"] + first
+            groups.append((first, [f"global_load_lds_dwordx4 {off[i]}, {base}"]))
     return groups
 
 
@@ -223,9 +211,8 @@ def check_rescale(uid, cb):
                 r = sreg(cb, h, u, i)
                 out.append(f"v_sub_f32_e32 v{r}, v{r}, {T[0]}")
         out.append("s_nop 15")                      # the MFMAs of the previous tile's PV have long finished; margin only
-        out.append(f"v_mul_f32_e32 {L[h]}, {L[h]}, {T[1]}")
-        for i in range(64):
-            a = f"a{64 * h + i}"
+        for i in range(64 + 16):
+            a = f"a{64 * h + i}" if i < 64 else lacc(h, i - 64)
             t = T[2 + (i & 3)]
             out.append(f"v_accvgpr_read_b32 {t}, {a}")
             out.append(f"v_mul_f32_e32 {t}, {t}, {T[1]}")
@@ -259,7 +246,8 @@ def pv_items(cb):
         rd = lambda frag, dt=dt, sfx=sfx: [f"ds_read_b64_tr_b16 {frag[1]}, {VA[0][dt]}{sfx}",
                                            f"ds_read_b64_tr_b16 {frag[2]}, {VA[1][dt]}{sfx}"]
         mf = lambda frag, u=u, t=t, dt=dt: [
-            f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)]
+            f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)] + (
+            [f"v_mfma_f32_32x32x16_bf16 {lacc(h)}, {ONES}, {ptup(cb, h, u, t)}, {lacc(h)}" for h in range(2)] if dt == 1 else [])
         items.append((rd, mf))
     return items
 
@@ -267,13 +255,21 @@ def pv_items(cb):
 def stream(out, items, valu_plan, extras=None, head=None, c0_zero=False):
     """Emits the fragment reads RING_DEPTH items ahead of the MFMAs that consume them.
     valu_plan: list of (first MFMA slot, last MFMA slot + 1, ops): ops are dealt evenly into the
-    slots (one slot follows each MFMA).  extras: {item index: [instruction groups]} placed after
-    that item's MFMAs.  head: instructions issued right after the first reads (they run while the
-    reads are in flight).  Waits are exact lgkmcnt values: LDS operations complete in order."""
+    slots (one slot follows each MFMA).  extras: {item index: (first, last)}: `first` is issued
+    before that item's MFMAs and `last` after them (an M0 write and the load that uses it).  head:
+    instructions issued right after the first reads (they run while the reads are in flight).
+    One wait covers two items; waits are exact lgkmcnt values (LDS operations complete in order)."""
     extras = extras or {}
-    n_slots = 2 * len(items)
+    mf_lists = []
+    for n, (rd, mf) in enumerate(items):
+        l = mf(ring(n))
+        if c0_zero:
+            l = [m.replace(f", {negm(0)}", ", 0").replace(f", {negm(1)}", ", 0") for m in l]
+        mf_lists.append(l)
+    n_slots = sum(len(l) for l in mf_lists)
     per_slot = [[] for _ in range(n_slots)]
     for (a, b, ops) in valu_plan:
+        assert b <= n_slots
         n = b - a
         base, rem = divmod(len(ops), n)
         k = 0
@@ -296,20 +292,20 @@ def stream(out, items, valu_plan, extras=None, head=None, c0_zero=False):
     if head:
         out.extend(head)
     slot = 0
-    for n, (rd, mf) in enumerate(items):
-        w = issued - 1 - last_id[n]
-        assert 0 <= w <= 15
-        out.append(f"s_waitcnt lgkmcnt({w})")
-        for mfma in mf(ring(n)):
-            if c0_zero:
-                mfma = mfma.replace(f", {negm(0)}", ", 0").replace(f", {negm(1)}", ", 0")
+    for n in range(len(items)):
+        if n % 2 == 0:
+            w = issued - 1 - last_id[min(n + 1, len(items) - 1)]
+            assert 0 <= w <= 15
+            out.append(f"s_waitcnt lgkmcnt({w})")
+        first, last = extras.get(n, ([], []))
+        out.extend(first)
+        for mfma in mf_lists[n]:
             out.append(mfma)
             out.extend(per_slot[slot])
             slot += 1
         if n + RING_DEPTH < len(items):
             issue_reads(n + RING_DEPTH)
-        for g in extras.get(n, []):
-            out.extend(g)
+        out.extend(last)
 
 
 # ---- program ------------------------------------------------------------------------------------
@@ -317,17 +313,17 @@ def prologue():
     out = []
     out += [f"v_mov_b32_e32 {NEG_INF}, 0xff800000", f"v_mov_b32_e32 {VPAD}, %[pad]", f"v_mov_b32_e32 {VLPM1}, %[lpm1]",
             f"v_mov_b32_e32 {MREL}, %[mrel]", f"v_mov_b32_e32 {JPL}, %[jpl]"]
-    for h in range(2):
-        out.append(f"v_mov_b32_e32 {L[h]}, 0")
-    for i in range(128):
+    for i in range(4):
+        out.append(f"v_mov_b32_e32 v{52 + i}, 0x3f803f80")
+    for i in list(range(128)) + list(range(192, 224)):
         out.append(f"v_accvgpr_write_b32 a{i}, 0")
     out += [f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_KEY0}, 0", f"s_mov_b32 {S_R0}, 0", f"s_mov_b32 {S_R1}, {SLOT}",
             f"s_mov_b32 {S_R2}, {2 * SLOT}", f"s_mov_b32 {S_R3}, {3 * SLOT}"]
     # tiles 0, 1, 2 -> slots 0, 1, 2; addresses of tile 3 prepared
     for slot in (S_R0, S_R1, S_R2):
         out += load_offset_ops()
-        for g in dma_ops(slot):
-            out += g
+        for first, last in dma_ops(slot):
+            out += first + ["s_nop 0"] + last
     out += load_offset_ops()
     out += [f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]          # tiles 0 and 1 have landed
     # QK(0) with C = 0, then m = row max of tile 0: -m tuples and S[0] -= m
@@ -353,13 +349,14 @@ def body(cb, masked):
     out = []
     nb = 1 - cb
     sm = softmax_ops(cb, masked)
-    yv = rowsum_ops(cb) + ["s_nop 7"] + rowmax_ops(nb) + load_offset_ops()
+    yv = rowmax_ops(nb) + load_offset_ops()
     items = qk_items(nb) + pv_items(cb)
     dma = dma_ops(S_R3)
-    extras = {1 + i: [dma[i]] for i in range(DMA_PER_TILE)}
+    extras = {17 + i: dma[i] for i in range(DMA_PER_TILE)}
     out += address_ops()
-    # P(h, u, t) is first read by PV item 4 (2u + t): the softmax may run 8 slots into the PV part
-    stream(out, items, [(0, 40, sm), (40, 64, yv)], extras, head=check_rescale(uid, cb))
+    # P(h, u, t) is first read by PV item 4 (2u + t): the softmax may run 12 slots into the PV part;
+    # the row max of S[nb] starts 12 MFMAs after the last QK MFMA
+    stream(out, items, [(0, 44, sm), (44, 72, yv)], extras, head=check_rescale(uid, cb))
     # ---- loop state; tile t+2 (issued one iteration ago) must have landed before the barrier
     out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_R3}",
             f"s_mov_b32 {S_R3}, {S_TMP}",
@@ -389,8 +386,7 @@ def epilogue():
     out = [".Lend_%=:", "s_nop 15", "s_nop 15"]
     out += [f"v_cmp_ne_u32_e32 vcc, 0, %[ok]", f"s_and_saveexec_b64 {S_SAVE}, vcc"]
     for h in range(2):
-        out += [f"v_mov_b32_e32 {T[7]}, {L[h]}", "s_nop 1", f"v_permlane32_swap_b32_e32 {L[h]}, {T[7]}", "s_nop 1",
-                f"v_add_f32_e32 {T[7]}, {L[h]}, {T[7]}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
+        out += [f"v_accvgpr_read_b32 {T[7]}, {lacc(h, 0)}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
         for dt in range(4):
             for g in range(4):
                 for e in range(4):
@@ -444,14 +440,14 @@ def main():
     text = "\n".join(f'        "{line}\\n"' for line in prog)
     qops = ", ".join(f'[q{h}{ks}] "a"(q[{h}][{ks}])' for h in range(2) for ks in range(8))
     vclob = ", ".join(f'"v{r}"' for r in range(24, 256))
-    aclob = ", ".join(f'"a{r}"' for r in range(0, 128))
+    aclob = ", ".join(f'"a{r}"' for r in list(range(0, 128)) + list(range(192, 224)))
     sclob = ", ".join(f'"s{r}"' for r in range(40, 56))
     tail = f'''
         :
         : [ka] "v"(A.ka), [val] "v"(A.val), [vah] "v"(A.vah), [jpl] "v"(A.jpl), [ch] "v"(A.ch),
           [mrel] "v"(A.mrel), [mlim] "v"(A.mlim), [o0] "v"(A.o0), [o1] "v"(A.o1), [ok] "v"(A.ok),
           [kb] "s"(A.kb), [vb] "s"(A.vb), [krb] "s"(A.krb), [vrb] "s"(A.vrb), [wrow] "s"(A.wrow),
-          [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm), [ones] "s"(0x3f803f80u),
+          [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm),
           {qops}
         : "memory", "vcc", "scc", "m0", {sclob},
           {vclob},

@@ -294,7 +294,15 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.lpm1 = uniform(Lp - 1);
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
+#if defined(MDX_ABL_NT1)
+    A.nt = 1;
+#endif
+#if defined(MDX_ABL_NOCORE)
+    if (A.nt == 12345) staircase_pair_core(A, q);
+    else if (row_ok) { A.o0[0] = q[0][0][0]; A.o1[0] = q[1][7][0]; }
+#else
     staircase_pair_core(A, q);
+#endif
 }
 
 }  // namespace
