@@ -20,30 +20,31 @@ Work of one wavefront: 32 query rows x 2 heads, keys in tiles of 64.
 Every K / V^T fragment feeds the MFMAs of both heads.  Register and key maps are those of
 attn_tile.h (key_of_reg, key_of_mfma_row).
 
-LDS: four slots of 32 KB (tile % 4), K rows then V rows, 256 bytes per row, filled by
+LDS: five slots of 32 KB (tile % 5), K rows then V rows, 256 bytes per row, filled by
 global_load_lds_dwordx4 (1 KB = 4 rows per instruction, 8 instructions per wavefront and tile).  The
 16-byte chunk c of row r sits at position c ^ (r % 16), which makes both fragment read patterns
 bank-conflict free without padding; the XOR shows up as one address register per k-step.
 
-Loop iteration t (S is double-buffered, cb = t & 1); the MFMA / fragment stream is continuous:
-  tile t+3: global -> LDS slot (issued early; it has two iterations to land)
-  X: 32 MFMAs of QK(t+1) -> S[1-cb]  ||  rescale check(t), P(t) = exp2(S[cb]) in place
-  Y: 32 MFMAs of PV(t) + 8 of ones . P^T (row sums)  ||  row max of S[1-cb], addresses of tile t+4,
-     loads of tile t+3
-  wait until tile t+2 has landed, barrier
+Loop iteration t (S is double-buffered, cb = t & 1).  The MFMA / fragment stream never drains: the
+reads of the first fragments of iteration t+1 are issued during the last items of iteration t.
+  items 0..15:  32 MFMAs of QK(t+1) -> S[1-cb]   ||  rescale check(t), P(t) = exp2(S[cb]) in place
+  wait until tile t+2 (loaded two iterations ago) has landed, barrier (publishes it; everyone has left tile t-1)
+  items 16..31: 32 MFMAs of PV(t) + 8 of ones . P^T (row sums)  ||  loads of tile t+4 -> slot of
+                tile t-1, row max of S[1-cb], fragment addresses of iteration t+1, addresses of tile t+5
 
-Physical registers (all clobbered; the compiler keeps v0..v23 and a128..a255 for the operands):
-  v24..v39  K / V^T fragment addresses   v40..v63  state, temporaries, load addresses
-  v64..v191 S[2][head][sub-tile][16]     v192..v223 -m tuples      v224..v247 fragment ring (6 x 4)
-  v248..v255 temporaries                 a0..a127  O^T[head][d tile][16]    a192..a223 row sums
-  s40..s55 loop state
+Physical registers (all clobbered; the compiler keeps v0..v15 and a128..a191, a224..a255 for operands):
+  v16..v23  temporaries                  v24..v39  K / V^T fragment addresses
+  v40..v63  state, ones, load addresses  v64..v191 S[2][head][sub-tile][16]
+  v192..v223 -m tuples                   v224..v255 fragment ring (8 x 4)
+  a0..a127  O^T[head][d tile][16]        a192..a223 row sums            s40..s55 loop state
 """
 import sys
 
 ROW = 256
 K_BYTES = 64 * ROW                 # 16384: K part of a slot; V part follows
 SLOT = 2 * K_BYTES
-RING_DEPTH = 5                     # fragments in flight
+RING_SLOTS = 8
+RING_DEPTH = 6                     # fragments in flight
 DMA_PER_TILE = 8                   # global_load_lds instructions per wavefront and tile
 
 # ---- register names ---------------------------------------------------------------------------
@@ -55,8 +56,9 @@ MX = ["v48", "v49"]
 MREL = "v50"
 GK = [f"v{56 + i}" for i in range(4)]            # global byte offsets of the rows the next loads fetch
 GV = [f"v{60 + i}" for i in range(4)]
-T = [f"v{248 + i}" for i in range(8)]
+T = [f"v{16 + i}" for i in range(8)]
 S_T, S_KEY0, S_R0, S_R1, S_R2, S_R3, S_TMP = "s40", "s41", "s42", "s43", "s44", "s45", "s46"
+S_R4 = "s51"
 S_SAVE = "s[48:49]"
 S_DST = "s50"
 
@@ -92,7 +94,7 @@ def lacc(h, i=None):
 
 
 def ring(i):
-    r = 224 + 4 * (i % 6)
+    r = 224 + 4 * (i % RING_SLOTS)
     return f"v[{r}:{r + 3}]", f"v[{r}:{r + 1}]", f"v[{r + 2}:{r + 3}]"
 
 
@@ -101,31 +103,29 @@ def key_const(u, i):
     return 32 * u + 16 * (i >> 3) + 4 * (i & 3) + ((i >> 2) & 1)
 
 
-def softmax_ops(cb, masked):
-    """S[cb] -> P in place, both heads, in the order PV consumes it.  Chunks of 8 values; the row
-    sums and the conversion of a chunk are issued one chunk after its exponentials (a v_exp result
-    needs a gap before a non-transcendental instruction reads it).  The row sums are not computed
-    here: the PV part multiplies P^T by a fragment of ones (8 MFMAs per tile instead of 64 adds;
-    the wavefront is bound by instruction issue, not by the matrix pipe)."""
-    ops = []
+def softmax_plan(cb, masked):
+    """S[cb] -> P in place, both heads, in the order PV consumes it, as {item: [ops]}.  Chunk c (8
+    values) is exponentiated during QK items 2c, 2c+1 (two values per MFMA) and converted during
+    items 2c+2, 2c+3 (a v_exp result needs a gap before another kind of instruction reads it), so
+    the last chunk is converted during the first two PV items; P(h, u, t) = chunk 2(2u + t) + h is
+    first read by PV item 4(2u + t).  The row sums are not computed here: the PV part multiplies
+    P^T by a fragment of ones (8 MFMAs per tile instead of 64 adds or 32 v_dot2, which executes on
+    the matrix pipe and stalls the MFMAs it is meant to hide behind)."""
+    plan = {n: [] for n in range(32)}
     chunks = [(h, u, t) for u in range(2) for t in range(2) for h in range(2)]
-    pending = None
-    for (h, u, t) in chunks:
-        regs = [sreg(cb, h, u, 8 * t + j) for j in range(8)]
-        if masked:
-            for j, r in enumerate(regs):
-                ops.append(f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}")
-                ops.append(f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]")
-                ops.append(f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc")
-        for r in regs:
-            ops.append(f"v_exp_f32_e32 v{r}, v{r}")
-        if pending:
-            ops += pending
+    for c, (h, u, t) in enumerate(chunks):
         base = sreg(cb, h, u, 8 * t)
-        pending = [f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}" for j in range(4)]
-    ops.append("s_nop 0")
-    ops += pending
-    return ops
+        for j in range(8):
+            item = 2 * c + (j >> 2)
+            r = base + j
+            if masked:
+                plan[item] += [f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}",
+                               f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]",
+                               f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc"]
+            plan[item].append(f"v_exp_f32_e32 v{r}, v{r}")
+        for j in range(4):
+            plan[2 * c + 2 + (j >> 1)].append(f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}")
+    return plan
 
 
 def rowmax_ops(b):
@@ -180,28 +180,34 @@ def dma_ops(slot_sreg):
     return groups
 
 
-def address_ops():
-    """Fragment addresses of this iteration: K of slot R1 (tile t+1), V of slot R0 (tile t)."""
-    ops = [f"v_add_u32_e32 {KA[0]}, {S_R1}, %[ka]"]
+def k_address_ops(slot_sreg):
+    """K fragment addresses (one per k-step: the swizzle is an XOR) for the slot in slot_sreg."""
+    ops = [f"v_add_u32_e32 {KA[0]}, {slot_sreg}, %[ka]"]
     for ks in range(1, 8):
         ops.append(f"v_xor_b32_e32 {KA[ks]}, {hex(ks << 5)}, {KA[0]}")
+    return ops
+
+
+def v_address_ops(slot_sreg):
+    """V^T fragment addresses (two rows x four d tiles) for the slot in slot_sreg."""
+    ops = []
     for q, name in enumerate(("%[val]", "%[vah]")):
-        ops.append(f"v_add_u32_e32 {VA[q][0]}, {S_R0}, {name}")
+        ops.append(f"v_add_u32_e32 {VA[q][0]}, {slot_sreg}, {name}")
         for dt in range(1, 4):
             ops.append(f"v_xor_b32_e32 {VA[q][dt]}, {hex(dt << 6)}, {VA[q][0]}")
     return ops
 
 
 def check_rescale(uid, cb):
-    """Lazy running-max update from MX = row max of S' = c s - m: only when some query exceeds the
-    stale max by more than 2^8.  The rare path moves m up by delta = max(MX, 0): the -m tuple and
-    the scores of tile t (computed with the old m) go down by delta, l and O^T (accumulation
-    registers) are scaled by 2^-delta."""
-    out = []
+    """Lazy running-max update from MX = row max of S' = c s - m: only when some query of either
+    head exceeds the stale max by more than 2^8.  The rare path moves m up by delta = max(MX, 0):
+    the -m tuple and the scores of tile t (computed with the old m) go down by delta, the row sums
+    and O^T (accumulation registers) are scaled by 2^-delta."""
+    lab = f".Lskip_{uid}_%="
+    out = [f"v_max_f32_e32 {T[0]}, {MX[0]}, {MX[1]}",
+           f"v_cmp_lt_f32_e32 vcc, 0x41000000, {T[0]}",
+           f"s_cbranch_vccz {lab}"]
     for h in range(2):
-        lab = f".Lskip_{uid}_{h}_%="
-        out.append(f"v_cmp_lt_f32_e32 vcc, 0x41000000, {MX[h]}")
-        out.append(f"s_cbranch_vccz {lab}")
         out.append(f"v_max_f32_e32 {T[0]}, 0, {MX[h]}")
         out.append(f"v_exp_f32_e64 {T[1]}, -{T[0]}")
         for i in range(16):
@@ -217,8 +223,8 @@ def check_rescale(uid, cb):
             out.append(f"v_accvgpr_read_b32 {t}, {a}")
             out.append(f"v_mul_f32_e32 {t}, {t}, {T[1]}")
             out.append(f"v_accvgpr_write_b32 {a}, {t}")
-        out.append("s_nop 7")
-        out.append(f"{lab}:")
+    out.append("s_nop 7")
+    out.append(f"{lab}:")
     return out
 
 
@@ -252,85 +258,71 @@ def pv_items(cb):
     return items
 
 
-def stream(out, items, valu_plan, extras=None, head=None, c0_zero=False):
-    """Emits the fragment reads RING_DEPTH items ahead of the MFMAs that consume them.
-    valu_plan: list of (first MFMA slot, last MFMA slot + 1, ops): ops are dealt evenly into the
-    slots (one slot follows each MFMA).  extras: {item index: (first, last)}: `first` is issued
-    before that item's MFMAs and `last` after them (an M0 write and the load that uses it).  head:
-    instructions issued right after the first reads (they run while the reads are in flight).
-    One wait covers two items; waits are exact lgkmcnt values (LDS operations complete in order)."""
-    extras = extras or {}
-    mf_lists = []
-    for n, (rd, mf) in enumerate(items):
-        l = mf(ring(n))
-        if c0_zero:
-            l = [m.replace(f", {negm(0)}", ", 0").replace(f", {negm(1)}", ", 0") for m in l]
-        mf_lists.append(l)
-    n_slots = sum(len(l) for l in mf_lists)
-    per_slot = [[] for _ in range(n_slots)]
-    for (a, b, ops) in valu_plan:
-        assert b <= n_slots
-        n = b - a
-        base, rem = divmod(len(ops), n)
-        k = 0
-        for i in range(n):
-            c = base + (1 if i < rem else 0)
-            per_slot[a + i] += ops[k:k + c]
-            k += c
-    issued = 0
-    last_id = {}
+class Ring:
+    """Issue order of the fragment reads and the exact lgkmcnt value that waits for one of them
+    (LDS operations of a wavefront complete in order; nothing else uses that counter here)."""
 
-    def issue_reads(n):
-        nonlocal issued
-        for r in items[n][0](ring(n)):
+    def __init__(self):
+        self.issued = 0
+        self.last = {}
+
+    def read(self, out, key, item, slot_index):
+        for r in item[0](ring(slot_index)):
             out.append(r)
-            issued += 1
-        last_id[n] = issued - 1
+            self.issued += 1
+        self.last[key] = self.issued - 1
 
-    for n in range(min(RING_DEPTH, len(items))):
-        issue_reads(n)
-    if head:
-        out.extend(head)
-    slot = 0
-    for n in range(len(items)):
-        if n % 2 == 0:
-            w = issued - 1 - last_id[min(n + 1, len(items) - 1)]
-            assert 0 <= w <= 15
-            out.append(f"s_waitcnt lgkmcnt({w})")
-        first, last = extras.get(n, ([], []))
-        out.extend(first)
-        for mfma in mf_lists[n]:
-            out.append(mfma)
-            out.extend(per_slot[slot])
-            slot += 1
-        if n + RING_DEPTH < len(items):
-            issue_reads(n + RING_DEPTH)
-        out.extend(last)
+    def wait(self, out, key):
+        w = self.issued - 1 - self.last[key]
+        assert 0 <= w <= 15, w
+        out.append(f"s_waitcnt lgkmcnt({w})")
 
 
-# ---- program ------------------------------------------------------------------------------------
+def spread(out, mfmas, valu):
+    """MFMAs of one item with its other instructions dealt evenly behind them."""
+    base, rem = divmod(len(valu), len(mfmas))
+    k = 0
+    for i, m in enumerate(mfmas):
+        out.append(m)
+        c = base + (1 if i < rem else 0)
+        out.extend(valu[k:k + c])
+        k += c
+
+
+def qk0_block(out):
+    """Prologue: QK(0) with C = 0 -> S[0]; drains its reads."""
+    items = qk_items(0)
+    rg = Ring()
+    for n in range(RING_DEPTH):
+        rg.read(out, n, items[n], n)
+    for n in range(16):
+        rg.wait(out, n)
+        for m in items[n][1](ring(n)):
+            out.append(m.replace(f", {negm(0)}", ", 0").replace(f", {negm(1)}", ", 0"))
+        if n + RING_DEPTH < 16:
+            rg.read(out, n + RING_DEPTH, items[n + RING_DEPTH], n + RING_DEPTH)
+
+
 def prologue():
     out = []
     out += [f"v_mov_b32_e32 {NEG_INF}, 0xff800000", f"v_mov_b32_e32 {VPAD}, %[pad]", f"v_mov_b32_e32 {VLPM1}, %[lpm1]",
             f"v_mov_b32_e32 {MREL}, %[mrel]", f"v_mov_b32_e32 {JPL}, %[jpl]"]
-    for i in range(4):
-        out.append(f"v_mov_b32_e32 v{52 + i}, 0x3f803f80")
-    for i in list(range(128)) + list(range(192, 224)):
-        out.append(f"v_accvgpr_write_b32 a{i}, 0")
     out += [f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_KEY0}, 0", f"s_mov_b32 {S_R0}, 0", f"s_mov_b32 {S_R1}, {SLOT}",
-            f"s_mov_b32 {S_R2}, {2 * SLOT}", f"s_mov_b32 {S_R3}, {3 * SLOT}"]
-    # tiles 0, 1, 2 -> slots 0, 1, 2; addresses of tile 3 prepared
-    for slot in (S_R0, S_R1, S_R2):
+            f"s_mov_b32 {S_R2}, {2 * SLOT}", f"s_mov_b32 {S_R3}, {3 * SLOT}", f"s_mov_b32 {S_R4}, {4 * SLOT}"]
+    # tiles 0..3 -> slots 0..3; addresses of tile 4 prepared
+    for slot in (S_R0, S_R1, S_R2, S_R3):
         out += load_offset_ops()
         for first, last in dma_ops(slot):
             out += first + ["s_nop 0"] + last
     out += load_offset_ops()
-    out += [f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]          # tiles 0 and 1 have landed
+    for i in range(4):
+        out.append(f"v_mov_b32_e32 v{52 + i}, 0x3f803f80")
+    for i in list(range(128)) + list(range(192, 224)):
+        out.append(f"v_accvgpr_write_b32 a{i}, 0")
+    out += [f"s_waitcnt vmcnt({2 * DMA_PER_TILE})", "s_barrier"]      # tiles 0 and 1 have landed
     # QK(0) with C = 0, then m = row max of tile 0: -m tuples and S[0] -= m
-    out.append(f"v_add_u32_e32 {KA[0]}, {S_R0}, %[ka]")
-    for ks in range(1, 8):
-        out.append(f"v_xor_b32_e32 {KA[ks]}, {hex(ks << 5)}, {KA[0]}")
-    stream(out, qk_items(0), [], c0_zero=True)
+    out += k_address_ops(S_R0)
+    qk0_block(out)
     out.append("s_nop 15")
     out += rowmax_ops(0)
     for h in range(2):
@@ -341,49 +333,78 @@ def prologue():
                 r = sreg(0, h, u, i)
                 out.append(f"v_sub_f32_e32 v{r}, v{r}, {MX[h]}")
         out.append(f"v_mov_b32_e32 {MX[h]}, 0")
+    # iteration 0 starts with its first K fragments (tile 1) in flight
+    out += k_address_ops(S_R1) + v_address_ops(S_R0)
+    items = qk_items(1)
+    for n in range(RING_DEPTH):
+        out += items[n][0](ring(n))
     return out
 
 
 def body(cb, masked):
+    """One iteration.  On entry the reads of items 0..RING_DEPTH-1 are in flight; on exit those of
+    the next iteration are."""
     uid = f"{cb}{int(masked)}"
     out = []
     nb = 1 - cb
-    sm = softmax_ops(cb, masked)
-    yv = rowmax_ops(nb) + load_offset_ops()
     items = qk_items(nb) + pv_items(cb)
-    dma = dma_ops(S_R3)
-    extras = {17 + i: dma[i] for i in range(DMA_PER_TILE)}
-    out += address_ops()
-    # P(h, u, t) is first read by PV item 4 (2u + t): the softmax may run 12 slots into the PV part;
-    # the row max of S[nb] starts 12 MFMAs after the last QK MFMA
-    stream(out, items, [(0, 44, sm), (44, 72, yv)], extras, head=check_rescale(uid, cb))
-    # ---- loop state; tile t+2 (issued one iteration ago) must have landed before the barrier
+    nxt = qk_items(cb)                                  # only their reads are used: first fragments of iteration t+1
+    plan = softmax_plan(cb, masked)
+    # second half: K addresses of tile t+2 (the K reads of this iteration were all issued by item 9),
+    # row max of S[nb] (complete after item 15), V^T addresses of tile t+1 (after the last V^T read
+    # of this iteration has been issued, item 25), addresses of the loads of tile t+4 (after the
+    # loads of tile t+3, items 17..24)
+    ka2 = k_address_ops(S_R2)
+    for i, op in enumerate(ka2):
+        plan[16 + i].append(op)
+    rm = rowmax_ops(nb)
+    per = -(-len(rm) // 8)
+    for i in range(8):
+        plan[18 + i] += rm[per * i:per * (i + 1)]
+    tail = v_address_ops(S_R1) + load_offset_ops()
+    per = -(-len(tail) // 6)
+    for i in range(6):
+        plan[26 + i] += tail[per * i:per * (i + 1)]
+    dma = dma_ops(S_R4)
+    rg = Ring()
+    for n in range(RING_DEPTH):
+        rg.last[n] = n
+    rg.issued = RING_DEPTH
+    out += check_rescale(uid, cb)
+    for n in range(32):
+        if n == 16:
+            # tile t+2 (loaded two iterations ago; tile t+3 may still be in flight) has landed; after
+            # the barrier every wavefront sees it and has left tile t-1, whose slot the loads below
+            # (tile t+4) overwrite
+            out += [f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]
+        if n % 2 == 0:
+            rg.wait(out, n + 1)
+        first, last = dma[n - 17] if 17 <= n < 17 + DMA_PER_TILE else ([], [])
+        out.extend(first)
+        spread(out, items[n][1](ring(n)), plan[n])
+        k = n + RING_DEPTH
+        rg.read(out, k, items[k] if k < 32 else nxt[k - 32], k)
+        out.extend(last)
     out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_R3}",
-            f"s_mov_b32 {S_R3}, {S_TMP}",
-            f"s_add_i32 {S_T}, {S_T}, 1", f"s_add_i32 {S_KEY0}, {S_KEY0}, 64", f"v_add_u32_e32 {MREL}, 64, {MREL}",
-            f"s_waitcnt vmcnt({DMA_PER_TILE}) lgkmcnt(0)", "s_barrier"]
+            f"s_mov_b32 {S_R3}, {S_R4}", f"s_mov_b32 {S_R4}, {S_TMP}",
+            f"s_add_i32 {S_T}, {S_T}, 1", f"s_add_i32 {S_KEY0}, {S_KEY0}, 64", f"v_add_u32_e32 {MREL}, 64, {MREL}"]
     return out
 
 
-def dispatch(cb):
-    """Chooses the masked or the plain body for tile t (wavefront-uniform)."""
-    out = [f".Ltop_{cb}_%=:",
-           f"s_cmp_ge_i32 {S_T}, %[nt]",
-           "s_cbranch_scc1 .Lend_%=",
-           f"s_cmp_lt_i32 {S_KEY0}, %[pad]",
-           f"s_cbranch_scc1 .Lbody_{cb}1_%=",
-           f"s_add_i32 {S_TMP}, {S_KEY0}, 64",
-           f"s_cmp_gt_i32 {S_TMP}, %[whm]",
-           f"s_cbranch_scc1 .Lbody_{cb}1_%="]
-    for masked in (False, True):
-        out.append(f".Lbody_{cb}{int(masked)}_%=:")
-        out += body(cb, masked)
-        out.append(f"s_branch .Ltop_{1 - cb}_%=")
-    return out
+def select(cb):
+    """Top of iteration t: leave after the last tile; tiles that need the key mask go out of line."""
+    return [f".Ltop_{cb}_%=:",
+            f"s_cmp_ge_i32 {S_T}, %[nt]",
+            "s_cbranch_scc1 .Lend_%=",
+            f"s_cmp_lt_i32 {S_KEY0}, %[pad]",
+            f"s_cbranch_scc1 .Lmasked_{cb}_%=",
+            f"s_add_i32 {S_TMP}, {S_KEY0}, 64",
+            f"s_cmp_gt_i32 {S_TMP}, %[whm]",
+            f"s_cbranch_scc1 .Lmasked_{cb}_%="]
 
 
 def epilogue():
-    out = [".Lend_%=:", "s_nop 15", "s_nop 15"]
+    out = [".Lend_%=:", "s_waitcnt lgkmcnt(0)", "s_nop 15", "s_nop 15"]
     out += [f"v_cmp_ne_u32_e32 vcc, 0, %[ok]", f"s_and_saveexec_b64 {S_SAVE}, vcc"]
     for h in range(2):
         out += [f"v_accvgpr_read_b32 {T[7]}, {lacc(h, 0)}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
@@ -395,16 +416,17 @@ def epilogue():
                     out.append(f"v_mul_f32_e32 {T[2 + e]}, {T[2 + e]}, {T[7]}")
                 out.append(f"v_cvt_pk_bf16_f32 {T[0]}, {T[2]}, {T[3]}")
                 out.append(f"v_cvt_pk_bf16_f32 {T[1]}, {T[4]}, {T[5]}")
-                out.append(f"global_store_dwordx2 %[o{h}], v[248:249], off offset:{(dt * 32 + 8 * g) * 2}")
-    out += [f"s_mov_b64 exec, {S_SAVE}", "s_waitcnt vmcnt(0)"]
+                out.append(f"global_store_dwordx2 %[o{h}], v[16:17], off offset:{(dt * 32 + 8 * g) * 2}")
+    out += [f"s_mov_b64 exec, {S_SAVE}"]
     return out
 
 
 def program():
+    # the common path falls through: top 0, plain body 0, top 1, plain body 1, one branch back
     out = prologue()
-    out.append("s_branch .Ltop_0_%=")
-    out += dispatch(0)
-    out += dispatch(1)
+    out += select(0) + body(0, False) + select(1) + body(1, False) + ["s_branch .Ltop_0_%="]
+    out += [".Lmasked_0_%=:"] + body(0, True) + ["s_branch .Ltop_1_%="]
+    out += [".Lmasked_1_%=:"] + body(1, True) + ["s_branch .Ltop_0_%="]
     out += epilogue()
     return out
 
@@ -439,7 +461,7 @@ def main():
     prog = program()
     text = "\n".join(f'        "{line}\\n"' for line in prog)
     qops = ", ".join(f'[q{h}{ks}] "a"(q[{h}][{ks}])' for h in range(2) for ks in range(8))
-    vclob = ", ".join(f'"v{r}"' for r in range(24, 256))
+    vclob = ", ".join(f'"v{r}"' for r in range(16, 256))
     aclob = ", ".join(f'"a{r}"' for r in list(range(0, 128)) + list(range(192, 224)))
     sclob = ", ".join(f'"s{r}"' for r in range(40, 56))
     tail = f'''

@@ -212,7 +212,10 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 // limit are fully masked.
 #include "staircase_pair_core.inc"
 
-constexpr int kPairSlots = 4;                     // LDS slots of one K tile + one V tile, 256-byte rows
+#if defined(MDX_ABL_DBG)
+__device__ unsigned mdx_dbg_buf[8192 * 4 * 8];
+#endif
+constexpr int kPairSlots = 5;                     // LDS slots of one K tile + one V tile, 256-byte rows
 constexpr int kPairLdsBytes = kPairSlots * 2 * kTileKeys * kRowBytes;
 
 // Values the asm reads from scalar registers must be wavefront-uniform in the compiler's eyes.
@@ -228,11 +231,15 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     extern __shared__ __attribute__((aligned(1024))) char lds_pair[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
-
     const int n_hslots = P.num_q_heads / 2;
-    const int hslot = blockIdx.x % n_hslots;
+
+    // One work item per workgroup: the dispatcher hands the next item to whichever CU frees up
+    // first, which balances the ragged item lengths (a fixed item -> CU assignment measured 10%
+    // slower although it saves the launch gap between two workgroups of a CU).
+    const int item = blockIdx.x;
+    const int hslot = item % n_hslots;
     int b, rg;
-    if (!locate_row_group(P, blockIdx.x / n_hslots, lane, b, rg)) return;
+    if (!locate_row_group(P, item / n_hslots, lane, b, rg)) return;
 
     const int seq0 = P.cu_seqlens[b];
     const int L = P.cu_seqlens[b + 1] - seq0;
@@ -294,6 +301,10 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.lpm1 = uniform(Lp - 1);
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
+#if defined(MDX_ABL_DBG)
+    A.dbg = mdx_dbg_buf + ((size_t)item * 4 + wave) * 8;
+    if (lane == 0) { mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 4] = A.nt; mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 5] = (unsigned)__builtin_amdgcn_s_memrealtime(); mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 6] = (unsigned)__builtin_amdgcn_s_memtime(); mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 7] = (unsigned)__builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11)); }
+#endif
 #if defined(MDX_ABL_NT1)
     A.nt = 1;
 #endif
@@ -307,6 +318,9 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
 
 }  // namespace
 
+#if defined(MDX_ABL_DBG)
+extern "C" int mdx_dbg_read(unsigned* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mdx_dbg_buf), (size_t)n * 4); }
+#endif
 extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                                          int64_t q_stride_t, int64_t q_stride_h,
                                          int64_t k_stride_t, int64_t k_stride_h,
