@@ -104,27 +104,48 @@ def key_const(u, i):
 
 
 def softmax_plan(cb, masked):
-    """S[cb] -> P in place, both heads, in the order PV consumes it, as {item: [ops]}.  Chunk c (8
-    values) is exponentiated during QK items 2c, 2c+1 (two values per MFMA) and converted during
-    items 2c+2, 2c+3 (a v_exp result needs a gap before another kind of instruction reads it), so
-    the last chunk is converted during the first two PV items; P(h, u, t) = chunk 2(2u + t) + h is
-    first read by PV item 4(2u + t).  The row sums are not computed here: the PV part multiplies
-    P^T by a fragment of ones (8 MFMAs per tile instead of 64 adds or 32 v_dot2, which executes on
-    the matrix pipe and stalls the MFMAs it is meant to hide behind)."""
+    """S[cb] -> P in place, both heads, in the order PV consumes it, as {item: [ops]}.
+    P(h, u, t) = chunk c = 2(2u + t) + h (8 values) is first read by PV item 16 + 4(2u + t).  The QK
+    items are the busy ones (two MFMAs, a fragment read and their share of these instructions have
+    to issue within the 65 cycles the two MFMAs execute), the PV items have room: chunks 0..5 are
+    exponentiated three values per QK item, chunks 6, 7 (read from item 28 on) during PV items
+    16..19; a chunk is converted at least one item after its last exponential (a v_exp result needs
+    a gap before another kind of instruction reads it), chunks 4..7 during PV items.  The row sums
+    are not computed here: the PV part multiplies P^T by a fragment of ones (8 MFMAs per tile
+    instead of 64 adds, or 32 v_dot2, which execute on the matrix pipe and stall the MFMAs they
+    are meant to hide behind)."""
     plan = {n: [] for n in range(32)}
     chunks = [(h, u, t) for u in range(2) for t in range(2) for h in range(2)]
-    for c, (h, u, t) in enumerate(chunks):
+
+    def exp_ops(c, j):
+        h, u, t = chunks[c]
+        r = sreg(cb, h, u, 8 * t + j)
+        ops = []
+        if masked:
+            ops += [f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}",
+                    f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]",
+                    f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc"]
+        return ops + [f"v_exp_f32_e32 v{r}, v{r}"]
+
+    def cvt_op(c, j):
+        h, u, t = chunks[c]
         base = sreg(cb, h, u, 8 * t)
-        for j in range(8):
-            item = 2 * c + (j >> 2)
-            r = base + j
-            if masked:
-                plan[item] += [f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}",
-                               f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]",
-                               f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc"]
-            plan[item].append(f"v_exp_f32_e32 v{r}, v{r}")
+        return f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}"
+
+    last_exp_item = {}
+    for e in range(48):                               # chunks 0..5: three values per QK item
+        c, j = e >> 3, e & 7
+        plan[e // 3] += exp_ops(c, j)
+        last_exp_item[c] = e // 3
+    for e in range(16):                               # chunks 6, 7: four values per item 16..19
+        c, j = 6 + (e >> 3), e & 7
+        plan[16 + e // 4] += exp_ops(c, j)
+        last_exp_item[c] = 16 + e // 4
+    for c in range(8):
+        first = {4: 16, 5: 17, 6: 20, 7: 21}.get(c, last_exp_item[c] + 1)
+        assert first > last_exp_item[c] and first + 1 < 16 + 4 * (c >> 1)
         for j in range(4):
-            plan[2 * c + 2 + (j >> 1)].append(f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}")
+            plan[first + (j >> 1)].append(cvt_op(c, j))
     return plan
 
 
