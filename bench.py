@@ -273,6 +273,7 @@ def main():
     torch.cuda.set_device(dev)
     K, W = args.steps, args.warmup
     result_ops = {}
+    calibration = None
 
     # A plain 1 GiB device copy: the yardstick against which FETCH_SIZE / WRITE_SIZE counter
     # readings of the kernels below are scaled when this command runs under rocprofv3 --pmc.
@@ -282,6 +283,16 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+        torch.cuda.empty_cache()
+        # What the matrix pipe sustains on this box: the clock is power-limited and operand bit
+        # toggling sets the power, so the library GEMM is timed on N(0,1) data and on zeros.
+        calibration = {}
+        for name, fill in (("gemm_bf16_8192_random", None), ("gemm_bf16_8192_zeros", 0.0)):
+            a_ = torch.randn(8192, 8192, device=dev).bfloat16() if fill is None else torch.zeros(8192, 8192, device=dev, dtype=torch.bfloat16)
+            b_ = a_.clone()
+            ms_, _ = time_kernel(lambda i: torch.matmul(a_, b_), 3, 10)
+            calibration[name] = dict(tflops=round(2 * 8192 ** 3 / ms_ / 1e9, 1), ms=round(ms_, 3))
+            del a_, b_
         torch.cuda.empty_cache()
 
     # ---------------- config 3: the step (store + staircase attention) -----------------------------
@@ -295,8 +306,8 @@ def main():
 
     o3 = torch.empty_like(g3["q"])
 
-    def attn_only(_):
-        q, k, v = g3["q"], g3["k"], g3["v"]
+    def attn_only(_, zeros=None):
+        q, k, v = zeros if zeros is not None else (g3["q"], g3["k"], g3["v"])
         rc = mdx.lib().mdx_staircase_attn_varlen(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o3.data_ptr(), q.stride(0), q.stride(1), k.stride(0), k.stride(1),
             v.stride(0), v.stride(1), o3.stride(0), o3.stride(1), g3["cu"].data_ptr(), g3["cu"].data_ptr(), len(host3["lens"]),
@@ -319,6 +330,14 @@ def main():
             ms=round(attn_ms, 4), ms_min=round(attn_min, 4), tflops=round(work3["flops"] / attn_ms / 1e9, 2),
             roofline=dict(bound="mfma", achieved=round(work3["flops"] / attn_ms / 1e9, 2), peak=PEAK_MFMA_TFLOPS,
                           unit="TFLOP/s", frac=round(work3["flops"] / attn_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), traffic=None))
+        if calibration is not None:
+            # the same launch on all-zero q/k/v (same strides): less bit toggling, higher clock
+            zf = torch.zeros(g3["q"].shape[0], (HQ + 2 * HKV) * D, dtype=torch.bfloat16, device=dev)
+            z = (torch.zeros_like(g3["q"]), torch.zeros_like(g3["k"]), zf[:, (HQ + HKV) * D:].view(-1, HKV, D))
+            z_ms, _ = time_kernel(lambda i: attn_only(i, z), 2, K)
+            calibration["staircase_attn_zero_inputs"] = dict(tflops=round(work3["flops"] / z_ms / 1e9, 1), ms=round(z_ms, 4))
+            del zf
+            del z
     if want("store"):
         # three rotating (source, cache) sets, about 900 MB touched per round trip, so the 256 MB
         # last-level cache cannot serve the next launch; the C ABI is called directly
@@ -450,6 +469,7 @@ def main():
         "roofline": result_ops.get("staircase_attn", {}).get("roofline"),
         "cpu_baseline": cpu,
         "ops": result_ops,
+        "calibration": calibration,
         "decode": decode,
         "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
     }
