@@ -174,7 +174,7 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8):
     cfg = DecoderConfig(num_layers=layers)
     model = Decoder(cfg, dev, seed=5)
     pages_per_seq = (1088 + new_tokens + PAGE - 1) // PAGE + 1
-    eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5)
+    eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5, decode_graphs=True, max_model_len=4096)
     g = torch.Generator().manual_seed(5)
     sp = SamplingParams(max_new_tokens=new_tokens, ignore_eos=True, transfer_count=S // steps_per_block)
     for _ in range(batch):

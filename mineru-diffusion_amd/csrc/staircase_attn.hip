@@ -212,9 +212,6 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 // limit are fully masked.
 #include "staircase_pair_core.inc"
 
-#if defined(MDX_ABL_DBG)
-__device__ unsigned mdx_dbg_buf[8192 * 4 * 8];
-#endif
 constexpr int kPairSlots = 5;                     // LDS slots of one K tile + one V tile, 256-byte rows
 constexpr int kPairLdsBytes = kPairSlots * 2 * kTileKeys * kRowBytes;
 
@@ -301,26 +298,11 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.lpm1 = uniform(Lp - 1);
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
-#if defined(MDX_ABL_DBG)
-    A.dbg = mdx_dbg_buf + ((size_t)item * 4 + wave) * 8;
-    if (lane == 0) { mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 4] = A.nt; mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 5] = (unsigned)__builtin_amdgcn_s_memrealtime(); mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 6] = (unsigned)__builtin_amdgcn_s_memtime(); mdx_dbg_buf[((size_t)item * 4 + wave) * 8 + 7] = (unsigned)__builtin_amdgcn_s_getreg(4 | (0 << 6) | (31 << 11)); }
-#endif
-#if defined(MDX_ABL_NT1)
-    A.nt = 1;
-#endif
-#if defined(MDX_ABL_NOCORE)
-    if (A.nt == 12345) staircase_pair_core(A, q);
-    else if (row_ok) { A.o0[0] = q[0][0][0]; A.o1[0] = q[1][7][0]; }
-#else
     staircase_pair_core(A, q);
-#endif
 }
 
 }  // namespace
 
-#if defined(MDX_ABL_DBG)
-extern "C" int mdx_dbg_read(unsigned* host, int n) { return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(mdx_dbg_buf), (size_t)n * 4); }
-#endif
 extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                                          int64_t q_stride_t, int64_t q_stride_h,
                                          int64_t k_stride_t, int64_t k_stride_h,

@@ -292,8 +292,12 @@ class BlockDiffusionEngine:
     model_runner.py:127-219), one GPU, eager."""
 
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
-                 max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None):
+                 max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
+                 decode_graphs: bool = False, max_model_len: int = 8192):
         self.model = model
+        self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
+        self.max_model_len = max_model_len
+        self._graphs = {}
         self.c = model.c
         self.device = model.lm_head.device
         self.max_num_batched_tokens = max_num_batched_tokens
@@ -407,6 +411,52 @@ class BlockDiffusionEngine:
                     block_tables=self._block_tables(seqs), block_size=S)
         return ids.to(dev, non_blocking=True), pos.to(dev, non_blocking=True)
 
+    # ---- decode graphs (model_runner.py:198-211 replay, :221-259 capture) ----
+    def _capture_decode(self, bs: int):
+        """Static input buffers + one captured forward of the decoder for `bs` sequences.  Every libmdx
+        launch goes to torch's current stream and allocates nothing itself, so the capture records
+        them like any torch op; page tables have their maximum width so that the split-KV launch
+        geometry is the same for every replay."""
+        S, dev = self.c.block_size, self.device
+        g = dict(ids=torch.zeros(bs, S, dtype=torch.int64, device=dev),
+                 pos=torch.zeros(bs, S, dtype=torch.int64, device=dev),
+                 slots=torch.full((bs, S), -1, dtype=torch.int32, device=dev),
+                 lens=torch.zeros(bs, dtype=torch.int32, device=dev),
+                 bt=torch.full((bs, (self.max_model_len + PAGE - 1) // PAGE), -1, dtype=torch.int32, device=dev))
+        set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                      # warm-up outside the capture (library handles, autotuning)
+            self.model(self.model.embed(g["ids"]), g["pos"])
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g["graph"] = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g["graph"]):
+            g["hidden"] = self.model(self.model.embed(g["ids"]), g["pos"])
+        torch.cuda.synchronize()
+        return g
+
+    def _run_decode_graph(self, seqs):
+        S, bs = self.c.block_size, len(seqs)
+        g = self._graphs.get(bs)
+        if g is None:
+            g = self._graphs[bs] = self._capture_decode(bs)
+        ids = torch.stack([s.current_denoising_block for s in seqs])
+        lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
+        pos = lens.unsqueeze(1) + torch.arange(S)
+        slots = torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32)
+        bt = torch.full(tuple(g["bt"].shape), -1, dtype=torch.int32)
+        for i, s in enumerate(seqs):
+            bt[i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
+        g["ids"].copy_(ids, non_blocking=True)
+        g["pos"].copy_(pos, non_blocking=True)
+        g["slots"].copy_(slots, non_blocking=True)
+        g["lens"].copy_((lens + S).to(torch.int32), non_blocking=True)
+        g["bt"].copy_(bt, non_blocking=True)
+        set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
+        g["graph"].replay()
+        return g["hidden"]
+
     def sample(self, logits, seqs) -> int:                 # layers/sampler.py:24-61 on the device
         sp = seqs[0].sampling_params
         if sp.denoising_strategy != "low_confidence_dynamic":
@@ -424,8 +474,11 @@ class BlockDiffusionEngine:
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
-        ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-        hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
+        if not is_prefill and self.decode_graphs and max(len(s) for s in seqs) + self.c.block_size <= self.max_model_len:
+            hidden = self._run_decode_graph(seqs)
+        else:
+            ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+            hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
         logits = self.model.compute_logits(hidden)
         if is_prefill:
             logits = logits.view(len(seqs), self.c.block_size, -1)
