@@ -201,6 +201,33 @@ int mdx_qk_norm_rope_store(const void* qkv, int64_t qkv_row_stride,
                            int64_t n_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                            int32_t dtype, mdx_stream_t stream);
 
+/*
+ * Residual add + RMSNorm of one decoder-layer input, one pass over the rows -- replaces
+ * RMSNorm.forward of engines/nano_dvlm/nanovllm/layers/layernorm.py:16-51 as called at
+ * nanovllm/models/sdar.py:147-152,180.
+ *
+ * x, out [rows, hidden]; weight [hidden]; row strides in elements.  With residual_in:
+ * s = float(x) + float(residual_in); residual_out = round(s); out = round(s * rsqrt(mean(s^2) +
+ * eps)) * weight, the product rounded again (add_rms_forward, :28-41).  With residual_in and
+ * residual_out both NULL: the same with s = float(x) (rms_forward, :16-26).  out may alias x and
+ * residual_out may alias residual_in.  Supported: MDX_BF16, hidden a multiple of 8 up to 8192.
+ */
+int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
+                     const void* residual_in, int64_t residual_in_row_stride,
+                     void* residual_out, int64_t residual_out_row_stride,
+                     const void* weight, float eps,
+                     void* out, int64_t out_row_stride,
+                     int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream);
+
+/*
+ * SiluAndMul.forward of engines/nano_dvlm/nanovllm/layers/activation.py:7-16 (called at
+ * nanovllm/models/sdar.py:110-111): x [rows, 2 * intermediate] -> out [rows, intermediate] =
+ * round(silu(float(x[:, :I]))) * x[:, I:], the product rounded again.  Row strides in
+ * elements.  Supported: MDX_BF16, intermediate a multiple of 8.
+ */
+int mdx_silu_and_mul(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride,
+                     int64_t rows, int32_t intermediate, int32_t dtype, mdx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -273,19 +273,37 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     const int hq = (int)((row / P.sq) % P.num_q_heads);
     const int b = (int)(row / P.sq / P.num_q_heads);
     const int ctx = P.context_lens[b];
+    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
     const int nv = (ctx + P.chunk - 1) / P.chunk;
     if (nv <= 1) return;                                   // written directly by the attention kernel
-    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
-    float M = kMinusBig;
-    for (int i = 0; i < nv; ++i) M = fmaxf(M, P.part_ml[((slot0 + i) * 2 + 0) * kMaxSq + s]);
-    float Lsum = 0.f;
+    // The kernel is a chain of memory latencies, not of bytes: every load of a group of four
+    // splits is issued before the first value is used.
+    float M = kMinusBig, Lsum = 0.f;
     float2 acc = make_float2(0.f, 0.f);
-    for (int i = 0; i < nv; ++i) {
-        const float w = __builtin_amdgcn_exp2f(P.part_ml[((slot0 + i) * 2 + 0) * kMaxSq + s] - M);
-        Lsum += w * P.part_ml[((slot0 + i) * 2 + 1) * kMaxSq + s];
-        const float2 po = *reinterpret_cast<const float2*>(P.part_o + ((slot0 + i) * kMaxSq + s) * kHeadDim + lane * 2);
-        acc.x += w * po.x;
-        acc.y += w * po.y;
+    for (int i0 = 0; i0 < nv; i0 += 4) {
+        float m[4], l[4];
+        float2 po[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t slot = slot0 + min(i0 + i, nv - 1);
+            m[i] = P.part_ml[(slot * 2 + 0) * kMaxSq + s];
+            l[i] = P.part_ml[(slot * 2 + 1) * kMaxSq + s];
+            po[i] = *reinterpret_cast<const float2*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + lane * 2);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
+        const float Mn = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), M);
+        const float keep = __builtin_amdgcn_exp2f(M - Mn);
+        Lsum *= keep; acc.x *= keep; acc.y *= keep;
+        M = Mn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool on = i0 + i < nv;
+            const float w = on ? __builtin_amdgcn_exp2f(m[i] - M) : 0.f;
+            Lsum += on ? w * l[i] : 0.f;
+            acc.x += on ? w * po[i].x : 0.f;
+            acc.y += on ? w * po[i].y : 0.f;
+        }
     }
     const float inv = 1.0f / Lsum;
     typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;

@@ -30,7 +30,7 @@ from torch import nn
 
 from .context import get_context, reset_context, set_context
 from .layers import Attention
-from .ops import flash_attn_with_kvcache, qk_norm_rope_store, sparse_attn_varlen, unmask_step
+from .ops import flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, silu_and_mul, sparse_attn_varlen, unmask_step
 
 PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
 
@@ -170,6 +170,7 @@ class DecoderConfig:
     block_size: int = 32
     mask_token_id: int = 151669
     fused_qk_rope_store: bool = True    # one libmdx launch for q/k norm + RoPE + KV store (else stock ops)
+    fused_layer_ops: bool = True        # libmdx residual-add + RMSNorm and SiLU-and-multiply (else stock ops)
 
 
 def _rms(x, w, eps):
@@ -191,14 +192,19 @@ class DecoderLayer(nn.Module):
         self.post_attention_layernorm = nn.Parameter(torch.ones(c.hidden_size))
         self.attn = Attention(c.num_heads, c.head_dim, c.head_dim ** -0.5, c.num_kv_heads)
 
+    def _norm(self, x, residual, w):
+        """layernorm.py:43-51: (normed, new residual)."""
+        c = self.c
+        if c.fused_layer_ops:
+            if residual is None:
+                return rms_norm(x, w, c.rms_norm_eps), x
+            return rms_norm(x, w, c.rms_norm_eps, residual)
+        residual = x if residual is None else x + residual
+        return _rms(residual, w, c.rms_norm_eps), residual
+
     def forward(self, positions, x, residual, cos, sin, cos_table=None, sin_table=None):
         c = self.c
-        if residual is None:                               # sdar.py:147-150
-            residual = x
-            h = _rms(x, self.input_layernorm, c.rms_norm_eps)
-        else:
-            residual = x + residual
-            h = _rms(residual, self.input_layernorm, c.rms_norm_eps)
+        h, residual = self._norm(x, residual, self.input_layernorm)       # sdar.py:147-150
         qkv = F.linear(h, self.qkv_proj)
         if c.fused_qk_rope_store:
             o = self._attend_fused(qkv, positions, cos_table, sin_table)
@@ -212,10 +218,14 @@ class DecoderLayer(nn.Module):
             q, k = _rope(q, cos, sin), _rope(k, cos, sin)
             o = self.attn(q, k, v)
         x = F.linear(o, self.o_proj)
-        residual = x + residual
-        h = _rms(residual, self.post_attention_layernorm, c.rms_norm_eps)
-        gate, up = F.linear(h, self.gate_up_proj).chunk(2, dim=-1)
-        return F.linear(F.silu(gate) * up, self.down_proj), residual
+        h, residual = self._norm(x, residual, self.post_attention_layernorm)
+        gate_up = F.linear(h, self.gate_up_proj)
+        if c.fused_layer_ops:
+            act = silu_and_mul(gate_up)
+        else:
+            gate, up = gate_up.chunk(2, dim=-1)
+            act = F.silu(gate) * up
+        return F.linear(act, self.down_proj), residual
 
 
     def _attend_fused(self, qkv, positions, cos_table, sin_table):
@@ -274,6 +284,8 @@ class Decoder(nn.Module):
         x, residual = inputs_embeds, None
         for layer in self.layers:
             x, residual = layer(positions, x, residual, cos, sin, self.cos, self.sin)
+        if self.c.fused_layer_ops:
+            return rms_norm(x, self.norm, self.c.rms_norm_eps, residual)[0]
         return _rms(x + residual, self.norm, self.c.rms_norm_eps)
 
     @torch.inference_mode()

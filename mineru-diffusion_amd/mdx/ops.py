@@ -104,6 +104,42 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     return q.view(*lead, num_q_heads, head_dim), None if k is None else k.view(*lead, num_kv_heads, head_dim), v
 
 
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
+    """RMSNorm.forward (nanovllm/layers/layernorm.py:43-51): returns the normed x, or with a
+    residual the pair (normed x + residual, x + residual), in one launch."""
+    _need_gpu(x, weight, residual)
+    hidden = x.shape[-1]
+    assert x.stride(-1) == 1 and weight.shape == (hidden,) and weight.dtype == x.dtype and weight.is_contiguous()
+    x2 = x.reshape(-1, hidden)
+    out = torch.empty((x2.shape[0], hidden), dtype=x.dtype, device=x.device)
+    r2 = r_out = None
+    if residual is not None:
+        assert residual.shape == x.shape and residual.dtype == x.dtype and residual.stride(-1) == 1
+        r2 = residual.reshape(-1, hidden)
+        r_out = torch.empty_like(out)
+    rc = _lib.lib().mdx_add_rms_norm(
+        x2.data_ptr(), x2.stride(0), r2.data_ptr() if r2 is not None else None, r2.stride(0) if r2 is not None else 0,
+        r_out.data_ptr() if r_out is not None else None, r_out.stride(0) if r_out is not None else 0,
+        weight.data_ptr(), float(eps), out.data_ptr(), out.stride(0), x2.shape[0], hidden, _DTYPES[x.dtype], _stream(x))
+    check(rc, "rms_norm")
+    if residual is None:
+        return out.view(x.shape)
+    return out.view(x.shape), r_out.view(x.shape)
+
+
+def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """SiluAndMul.forward (nanovllm/layers/activation.py:13-16): x [..., 2I] -> silu(x[..., :I]) * x[..., I:]."""
+    _need_gpu(x)
+    assert x.shape[-1] % 2 == 0 and x.stride(-1) == 1
+    inter = x.shape[-1] // 2
+    x2 = x.reshape(-1, 2 * inter)
+    out = torch.empty((x2.shape[0], inter), dtype=x.dtype, device=x.device)
+    rc = _lib.lib().mdx_silu_and_mul(x2.data_ptr(), x2.stride(0), out.data_ptr(), out.stride(0), x2.shape[0], inter,
+                                     _DTYPES[x.dtype], _stream(x))
+    check(rc, "silu_and_mul")
+    return out.view(*x.shape[:-1], inter)
+
+
 # --------------------------------------------------------------------------- staircase prefill
 def sparse_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor,
                        cu_seqlens_k: torch.Tensor, staircase_size: int = 4, *, max_seqlen: int | None = None,

@@ -31,6 +31,10 @@ select_transfer             torch.topk on tie-free inputs, brute force over all
 slot_of / get_slots         brute force token-by-token formula
 rms_norm_ref / rope_ref     unit RMS after norm, F.rms_norm, rotation preserves pair norms,
                             position 0 is the identity, complex-multiplication form
+add_rms_norm                residual is the rounded sum; reduces to rms_norm_ref for a zero residual;
+                            F.rms_norm of the fp32 sum; variance taken before the rounding (a case
+                            where the two differ)
+silu_and_mul                F.silu * other half; silu(0) = 0, silu(x) -> x and -> 0 in the tails
 dense_forward               built from the pinned attention oracle and plain matmuls; its mask
                             and SDPA are the functions above
 ==========================  =====================================================
@@ -49,4 +53,4 @@ from .kvstore import store_kvcache  # noqa: F401
 from .unmask import confidence_argmax, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
 from .slots import slot_of, get_slots  # noqa: F401
 from .engine import dense_forward, expected_passes  # noqa: F401
-from .fused import qk_norm_rope, rms_norm_ref, rope_ref  # noqa: F401
+from .fused import qk_norm_rope, rms_norm_ref, rope_ref, add_rms_norm, silu_and_mul  # noqa: F401

@@ -47,3 +47,42 @@ def test_qk_norm_rope_splits_heads_q_k_v():
     assert torch.equal(v, qkv[:, (hq + hkv) * d:].view(N, hkv, d))
     assert torch.allclose(q.float().pow(2).mean(-1), torch.ones(N, hq), atol=2e-2)
     assert torch.equal(k[2, 1], oracle.rms_norm_ref(qkv[2, (hq + 1) * d:(hq + 2) * d], torch.ones(d).bfloat16(), 1e-6))
+
+
+def test_add_rms_norm_rounds_the_residual_but_not_the_variance():
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(6, 256, generator=g) * 3).bfloat16()
+    r = (torch.randn(6, 256, generator=g) * 3).bfloat16()
+    w = (torch.rand(256, generator=g) + 0.5).bfloat16()
+    y, nr = oracle.add_rms_norm(x, r, w, 1e-6)
+    s = x.float() + r.float()                                   # exact in fp32 for bf16 operands of similar size
+    assert torch.equal(nr, s.bfloat16())
+    assert torch.allclose(y.float(), F.rms_norm(s, (256,), w.float(), 1e-6), rtol=2 ** -6, atol=1e-3)
+    # a zero residual reduces it to the plain norm, bit for bit
+    y0, nr0 = oracle.add_rms_norm(x, torch.zeros_like(x), w, 1e-6)
+    assert torch.equal(y0, oracle.rms_norm_ref(x, w, 1e-6)) and torch.equal(nr0, x)
+    assert oracle.add_rms_norm(x, None, w, 1e-6)[1] is None
+    # the mean of squares is taken over the unrounded sum: 256 + 1 rounds to 256 in bf16, and the
+    # row [257, 0, ...] must normalise with 257, not 256
+    x1 = torch.zeros(1, 8).bfloat16(); x1[0, 0] = 256.0
+    r1 = torch.zeros(1, 8).bfloat16(); r1[0, 0] = 1.0
+    y1, nr1 = oracle.add_rms_norm(x1, r1, torch.ones(8).bfloat16(), 0.0)
+    assert nr1[0, 0].item() == 256.0                            # the stored residual lost the 1
+    assert y1[0, 0].item() == torch.tensor(257.0 / (257.0 / 8 ** 0.5)).bfloat16().item()   # = sqrt(8) either way here
+    x2 = torch.tensor([[256.0, 128.0] + [0.0] * 6]).bfloat16()
+    r2 = torch.tensor([[1.0, 0.0] + [0.0] * 6]).bfloat16()
+    y2, _ = oracle.add_rms_norm(x2, r2, torch.ones(8).bfloat16(), 0.0)
+    rms_unrounded = ((257.0 ** 2 + 128.0 ** 2) / 8) ** 0.5
+    assert y2[0, 1].item() == torch.tensor(128.0 / rms_unrounded).bfloat16().item()
+
+
+def test_silu_and_mul_closed_forms():
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(5, 64, generator=g) * 3).bfloat16()
+    y = oracle.silu_and_mul(x)
+    assert y.shape == (5, 32)
+    assert torch.equal(y, F.silu(x[:, :32]) * x[:, 32:])        # the library routine, same rounding points
+    t = torch.tensor([[0.0, 30.0, -30.0, 1.0, 1.0, 2.0, 2.0, 2.0]]).bfloat16()
+    yt = oracle.silu_and_mul(t)
+    assert yt[0, 0].item() == 0.0 and yt[0, 1].item() == 60.0 and abs(yt[0, 2].item()) < 1e-10
+    assert abs(yt[0, 3].item() - 2 * 0.7310585786) < 2e-2       # silu(1) = 1 / (1 + e^-1)
