@@ -83,6 +83,7 @@ class Sequence:
         self.current_denoising_block = torch.full((denoising_block_size,), mask_token_id, dtype=torch.int64)
         self.current_step_map = torch.zeros((denoising_block_size,), dtype=torch.int32)
         self.current_denoise_step = 0
+        self.block_has_mask = None                       # filled by the engine's sampler; see postprocess
 
     def __len__(self):
         return self.num_tokens
@@ -310,6 +311,7 @@ class BlockDiffusionEngine:
         self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
         self.max_model_len = max_model_len
         self._graphs = {}
+        self._temps = None
         self.c = model.c
         self.device = model.lm_head.device
         self.max_num_batched_tokens = max_num_batched_tokens
@@ -362,7 +364,12 @@ class BlockDiffusionEngine:
     def postprocess(self, seqs):                           # scheduler.py:65-82
         for seq in seqs:
             if not seq.is_caching:
-                if not (seq.current_denoising_block == seq.mask_token_id).any():
+                probe = seq.block_has_mask                  # (block tensor, any mask left) noted by `sample`
+                if probe is not None and probe[0] is seq.current_denoising_block:
+                    masked = probe[1]
+                else:
+                    masked = bool((seq.current_denoising_block == seq.mask_token_id).any())
+                if not masked:
                     seq.status = SequenceStatus.CACHING
                 continue
             finished = any((seq.current_denoising_block == s).any() for s in seq.sampling_params.stop_token_ids)
@@ -428,13 +435,27 @@ class BlockDiffusionEngine:
         """Static input buffers + one captured forward of the decoder for `bs` sequences.  Every libmdx
         launch goes to torch's current stream and allocates nothing itself, so the capture records
         them like any torch op; page tables have their maximum width so that the split-KV launch
-        geometry is the same for every replay."""
+        geometry is the same for every replay.  The five inputs are views into one device buffer
+        that mirrors one pinned host buffer: a pass uploads them with a single copy."""
         S, dev = self.c.block_size, self.device
-        g = dict(ids=torch.zeros(bs, S, dtype=torch.int64, device=dev),
-                 pos=torch.zeros(bs, S, dtype=torch.int64, device=dev),
-                 slots=torch.full((bs, S), -1, dtype=torch.int32, device=dev),
-                 lens=torch.zeros(bs, dtype=torch.int32, device=dev),
-                 bt=torch.full((bs, (self.max_model_len + PAGE - 1) // PAGE), -1, dtype=torch.int32, device=dev))
+        width = (self.max_model_len + PAGE - 1) // PAGE
+        fields = [("ids", torch.int64, (bs, S)), ("pos", torch.int64, (bs, S)), ("slots", torch.int32, (bs, S)),
+                  ("lens", torch.int32, (bs,)), ("bt", torch.int32, (bs, width))]
+        offsets, at = {}, 0
+        for name, dt, shape in fields:
+            offsets[name] = at
+            at += (math.prod(shape) * dt.itemsize + 15) // 16 * 16
+        g = dict(dev_buf=torch.zeros(at, dtype=torch.uint8, device=dev),
+                 pin_buf=torch.zeros(at, dtype=torch.uint8, pin_memory=True), host={})
+        for name, dt, shape in fields:
+            n = math.prod(shape) * dt.itemsize
+            g[name] = g["dev_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
+            g["host"][name] = g["pin_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
+        g["host"]["slots"].fill_(-1)
+        g["host"]["bt"].fill_(-1)
+        g["dev_buf"].copy_(g["pin_buf"])
+        g["result"] = torch.zeros(2, bs, S, dtype=torch.int64, device=dev)          # tokens, transfer flags
+        g["result_host"] = torch.zeros(2, bs, S, dtype=torch.int64, pin_memory=True)
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -449,46 +470,88 @@ class BlockDiffusionEngine:
         return g
 
     def _run_decode_graph(self, seqs):
+        """Uploads the pass inputs (one copy) and replays the graph.  Within a denoising block
+        nothing has to be uploaded at all: lengths, slots and page tables are those of the previous
+        pass, and the token block on the device is the one the unmask step just updated in place
+        (the host rows handed to the sequences by `sample` are a download of exactly that buffer)."""
         S, bs = self.c.block_size, len(seqs)
         g = self._graphs.get(bs)
         if g is None:
             g = self._graphs[bs] = self._capture_decode(bs)
-        ids = torch.stack([s.current_denoising_block for s in seqs])
-        lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
-        pos = lens.unsqueeze(1) + torch.arange(S)
-        slots = torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32)
-        bt = torch.full(tuple(g["bt"].shape), -1, dtype=torch.int32)
-        for i, s in enumerate(seqs):
-            bt[i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
-        g["ids"].copy_(ids, non_blocking=True)
-        g["pos"].copy_(pos, non_blocking=True)
-        g["slots"].copy_(slots, non_blocking=True)
-        g["lens"].copy_((lens + S).to(torch.int32), non_blocking=True)
-        g["bt"].copy_(bt, non_blocking=True)
+        signature = [(s.seq_id, s.num_tokens, len(s.block_table)) for s in seqs]
+        rows = g.get("rows")
+        fresh = (g.get("signature") == signature and rows is not None
+                 and all(s.current_denoising_block is r for s, r in zip(seqs, rows)))
+        if not fresh:
+            h = g["host"]
+            torch.stack([s.current_denoising_block for s in seqs], out=h["ids"])
+            lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
+            torch.add(lens.unsqueeze(1), torch.arange(S), out=h["pos"])
+            h["slots"].copy_(torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32))
+            h["lens"].copy_(lens + S)
+            h["bt"].fill_(-1)
+            for i, s in enumerate(seqs):
+                h["bt"][i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
+            g["dev_buf"].copy_(g["pin_buf"], non_blocking=True)
+            g["signature"] = signature
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
         g["graph"].replay()
-        return g["hidden"]
+        return g["hidden"], g
 
-    def sample(self, logits, seqs) -> int:                 # layers/sampler.py:24-61 on the device
+    def _temperatures(self, seqs):
+        key = tuple(s.temperature for s in seqs)
+        if self._temps is None or self._temps[0] != key:
+            self._temps = (key, torch.tensor(key, dtype=torch.float32, device=self.device))
+        return self._temps[1]
+
+    def sample(self, logits, seqs, g=None) -> int:         # layers/sampler.py:24-61 on the device
+        """Unmask step on the device, then one download of (tokens, transfer flags).  With the
+        buffers `g` of a decode graph, the token block is the graph's own input buffer (already
+        on the device) and the download goes through one pinned buffer."""
         sp = seqs[0].sampling_params
         if sp.denoising_strategy != "low_confidence_dynamic":
             raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
-        x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
-        temps = torch.tensor([s.temperature for s in seqs], dtype=torch.float32, device=self.device)
-        _, _, transfer, count = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
-                                            temperatures=temps)
-        x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
-        for i, s in enumerate(seqs):
-            s.current_denoising_block = x_cpu[i]
-            s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
+        if g is not None:
+            x = g["ids"]
+        else:
+            x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
+        _, _, transfer, _n = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
+                                         temperatures=self._temperatures(seqs))
+        if g is None:
+            x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
+            for i, s in enumerate(seqs):
+                s.current_denoising_block = x_cpu[i]
+                s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
+                s.current_denoise_step += 1
+            return int(transfer_cpu.sum().item())
+        g["result"][0].copy_(x)
+        g["result"][1].copy_(transfer)
+        g["result_host"].copy_(g["result"], non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        x_cpu, transfer_cpu = g["result_host"][0].clone(), g["result_host"][1].bool()
+        # one indexed write for all step maps: the sequences' maps are rows of one batch tensor
+        maps, map_rows = g.get("maps"), g.get("map_rows")
+        if maps is None or not all(s.current_step_map is r for s, r in zip(seqs, map_rows)):
+            maps = g["maps"] = torch.stack([s.current_step_map for s in seqs])
+            map_rows = g["map_rows"] = list(maps.unbind(0))
+            for s, r in zip(seqs, map_rows):
+                s.current_step_map = r
+        steps = torch.tensor([s.current_denoise_step for s in seqs], dtype=torch.int32)
+        maps[transfer_cpu] = steps.unsqueeze(1).expand_as(maps)[transfer_cpu]
+        rows = g["rows"] = list(x_cpu.unbind(0))
+        has_mask = (x_cpu == seqs[0].mask_token_id).any(1).tolist()
+        for s, r, m in zip(seqs, rows, has_mask):
+            s.current_denoising_block = r
+            s.block_has_mask = (r, m)
             s.current_denoise_step += 1
-        return int(count.sum().item())
+        return int(transfer_cpu.sum().item())
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
         if not is_prefill and self.decode_graphs and max(len(s) for s in seqs) + self.c.block_size <= self.max_model_len:
-            hidden = self._run_decode_graph(seqs)
+            hidden, g = self._run_decode_graph(seqs)
         else:
+            g = None
             ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
             hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
         logits = self.model.compute_logits(hidden)
@@ -496,7 +559,7 @@ class BlockDiffusionEngine:
             logits = logits.view(len(seqs), self.c.block_size, -1)
         if self.on_logits is not None:
             self.on_logits(is_prefill, seqs, logits)
-        n = self.sample(logits, seqs)
+        n = self.sample(logits, seqs, g)
         reset_context()
         return n
 

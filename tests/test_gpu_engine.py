@@ -100,7 +100,7 @@ def test_decode_graph_replays_match_eager(dev):
             blk = torch.full((32,), cfg.mask_token_id, dtype=torch.int64)
             blk[: 4 * rep] = torch.randint(0, 900, (4 * rep,), generator=g)
             s.current_denoising_block = blk
-        hidden = eng._run_decode_graph(seqs).clone()
+        hidden = eng._run_decode_graph(seqs)[0].clone()
         torch.cuda.synchronize()
         ids, pos = eng.prepare_decode(seqs)                # eager, its own context tensors
         gr = eng._graphs[len(seqs)]
