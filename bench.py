@@ -165,7 +165,7 @@ def make_cfg4(dev, n_sets=2, seed=4):
 
 
 # ----------------------------------------------------------------------------- config 5
-def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8):
+def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, masked_rows_only=True):
     """Random-init SDAR-shaped decoder (28 layers, hidden 2048, Hq 16 / Hkv 8 / d 128, SwiGLU 6144,
     vocab 151936), batch 32, 1024 random prefix embeddings + 64 prompt tokens per sequence, 2048 new
     tokens in 32-token blocks, k = 32/8 = 4 committed positions per denoising pass, threshold 0.9.
@@ -175,7 +175,8 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8):
     cfg = DecoderConfig(num_layers=layers)
     model = Decoder(cfg, dev, seed=5)
     pages_per_seq = (1088 + new_tokens + PAGE - 1) // PAGE + 1
-    eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5, decode_graphs=True, max_model_len=4096)
+    eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5, decode_graphs=True, max_model_len=4096,
+                               masked_rows_only=masked_rows_only)
     g = torch.Generator().manual_seed(5)
     prompts = []
     for _ in range(batch):
@@ -203,6 +204,8 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8):
                prefill_passes=st["prefill_passes"], decode_passes=st["decode_passes"],
                prefill_s=round(st["prefill_s"], 3), decode_s=round(st["decode_s"], 3),
                ms_per_decode_pass=round(st["decode_s"] / max(1, st["decode_passes"]) * 1e3, 3), layers=layers,
+               vocabulary_projection=("rows of still-masked positions only (the unmask rule reads no others; same tokens)"
+                                      if masked_rows_only else "all 32 positions of every block, as the reference computes them"),
                model="random-init 28-layer SDAR-shaped decoder, stock PyTorch-ROCm GEMMs, libmdx attention/KV store/unmask")
     del eng, model
     torch.cuda.empty_cache()
@@ -447,6 +450,8 @@ def main():
         del g3, attn
         torch.cuda.empty_cache()
         decode = run_cfg5(dev)
+        full = run_cfg5(dev, masked_rows_only=False)
+        decode["with_full_logits"] = {k: full[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass", "vocabulary_projection")}
 
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
     cpu = None

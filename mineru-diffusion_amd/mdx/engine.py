@@ -30,7 +30,8 @@ from torch import nn
 
 from .context import get_context, reset_context, set_context
 from .layers import Attention
-from .ops import flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, silu_and_mul, sparse_attn_varlen, unmask_step
+from .ops import (confidence_argmax, flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
+                  sparse_attn_varlen, unmask_step)
 
 PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
 
@@ -306,10 +307,11 @@ class BlockDiffusionEngine:
 
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
                  max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
-                 decode_graphs: bool = False, max_model_len: int = 8192):
+                 decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True):
         self.model = model
         self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
         self.max_model_len = max_model_len
+        self.masked_rows_only = masked_rows_only           # graph decode: logits for still-masked positions only
         self._graphs = {}
         self._temps = None
         self.c = model.c
@@ -494,6 +496,7 @@ class BlockDiffusionEngine:
                 h["bt"][i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
             g["dev_buf"].copy_(g["pin_buf"], non_blocking=True)
             g["signature"] = signature
+            g["x_host"] = h["ids"]                          # host copy of the device token blocks
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
         g["graph"].replay()
         return g["hidden"], g
@@ -524,11 +527,17 @@ class BlockDiffusionEngine:
                 s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
                 s.current_denoise_step += 1
             return int(transfer_cpu.sum().item())
+        return self._download(seqs, g, x, transfer)
+
+    def _download(self, seqs, g, x, transfer) -> int:
+        """One download of (tokens, transfer flags) through the pinned buffer, then the per-sequence
+        bookkeeping of sampler.py:56-59 as batch operations."""
         g["result"][0].copy_(x)
         g["result"][1].copy_(transfer)
         g["result_host"].copy_(g["result"], non_blocking=True)
         torch.cuda.current_stream().synchronize()
         x_cpu, transfer_cpu = g["result_host"][0].clone(), g["result_host"][1].bool()
+        g["x_host"] = x_cpu
         # one indexed write for all step maps: the sequences' maps are rows of one batch tensor
         maps, map_rows = g.get("maps"), g.get("map_rows")
         if maps is None or not all(s.current_step_map is r for s, r in zip(seqs, map_rows)):
@@ -546,6 +555,38 @@ class BlockDiffusionEngine:
             s.current_denoise_step += 1
         return int(transfer_cpu.sum().item())
 
+    def _sample_masked_rows(self, hidden, seqs, g) -> int:
+        """The unmask step restricted to the positions that are still masked.  The selection reads
+        confidences of masked positions only (sampler.py:39) and commits x0 only there (:54), so the
+        logits of committed positions are never looked at: the vocabulary projection, the softmax
+        and the argmax run on the masked rows alone (half the rows on average, none in the pass
+        that only caches a finished block), with identical results."""
+        sp = seqs[0].sampling_params
+        if sp.denoising_strategy != "low_confidence_dynamic":
+            raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
+        S, bs, mask_id = self.c.block_size, len(seqs), seqs[0].mask_token_id
+        idx = (g["x_host"].view(-1) == mask_id).nonzero().squeeze(1)
+        if idx.numel() == 0:
+            for s in seqs:
+                s.current_denoise_step += 1
+            return 0
+        idx_dev = idx.to(self.device, non_blocking=True)
+        logits = F.linear(hidden.view(bs * S, -1).index_select(0, idx_dev), self.model.lm_head)
+        temps = self._temperatures(seqs)
+        if len(set(self._temps[0])) == 1:
+            temps = temps[:1]
+        else:
+            temps = temps.index_select(0, idx_dev // S)
+        x0_rows, p_rows = confidence_argmax(logits, temps)
+        if "x0" not in g:
+            g["x0"] = torch.zeros(bs * S, dtype=torch.int64, device=self.device)
+            g["x0_p"] = torch.zeros(bs * S, dtype=torch.float32, device=self.device)
+        g["x0"].index_copy_(0, idx_dev, x0_rows)
+        g["x0_p"].index_copy_(0, idx_dev, p_rows)
+        transfer, _n = select_transfer(g["x0"].view(bs, S), g["x0_p"].view(bs, S), g["ids"], mask_id,
+                                       sp.dynamic_threshold, sp.transfer_count)
+        return self._download(seqs, g, g["ids"], transfer)
+
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
         if not is_prefill and self.decode_graphs and max(len(s) for s in seqs) + self.c.block_size <= self.max_model_len:
@@ -554,6 +595,10 @@ class BlockDiffusionEngine:
             g = None
             ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
             hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
+        if g is not None and self.masked_rows_only and self.on_logits is None and self.unmask is unmask_step:
+            n = self._sample_masked_rows(hidden, seqs, g)
+            reset_context()
+            return n
         logits = self.model.compute_logits(hidden)
         if is_prefill:
             logits = logits.view(len(seqs), self.c.block_size, -1)

@@ -129,3 +129,28 @@ def test_engine_with_decode_graphs_generates_like_eager(dev):
     # same kernels; only the split-KV geometry may differ (page table width), which can flip a near-tie
     same = sum(int(a == b) for a, b in zip(*outs))
     assert same >= 60, f"only {same}/64 tokens agree"
+
+
+@pytest.mark.parametrize("temps", [(1.0, 1.0, 1.0), (1.0, 0.7, 1.3)])
+def test_masked_rows_only_sampling_matches_full_logits(dev, temps):
+    """Graph decode with the vocabulary projection and the unmask step restricted to the still
+    masked positions vs the same engine on full [bs, 32, V] logits: same committed tokens and step
+    maps (the projection runs on fewer rows, which may pick another GEMM tiling and flip a near-tie)."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for rows_only in (False, True):
+        eng = BlockDiffusionEngine(model, num_pages=16, shuffle_pages_seed=3, decode_graphs=True, max_model_len=1024,
+                                   masked_rows_only=rows_only)
+        g = torch.Generator().manual_seed(2)
+        seqs = [eng.add_request(torch.randint(0, 900, (n,), generator=g).tolist(),
+                                SamplingParams(max_new_tokens=96, ignore_eos=True, transfer_count=4, temperature=t))
+                for n, t in zip((290, 33, 150), temps)]
+        eng.generate()
+        outs.append([(s.completion_token_ids, list(s.step_map)) for s in seqs])
+        assert eng.stats["decode_passes"] == 3 * 9 - 1      # 3 blocks x (8 denoise + 1 caching pass); the prefill pass is the first denoise
+    for (ta, ma), (tb, mb) in zip(*outs):
+        assert len(ta) == len(tb) == 96 and len(ma) == len(mb)
+        same = sum(int(a == b) for a, b in zip(ta, tb))
+        assert same >= 90, f"only {same}/96 tokens agree"
+        assert sum(int(a == b) for a, b in zip(ma, mb)) >= 90
