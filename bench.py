@@ -273,6 +273,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
+    ap.add_argument("--no-full-logits-leg", action="store_true",
+                    help="decode leg: skip the second generation that projects all 32 positions of every block")
     ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,decode (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -450,8 +452,9 @@ def main():
         del g3, attn
         torch.cuda.empty_cache()
         decode = run_cfg5(dev)
-        full = run_cfg5(dev, masked_rows_only=False)
-        decode["with_full_logits"] = {k: full[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass", "vocabulary_projection")}
+        if not args.no_full_logits_leg:
+            full = run_cfg5(dev, masked_rows_only=False)
+            decode["with_full_logits"] = {k: full[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass", "vocabulary_projection")}
 
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
     cpu = None
