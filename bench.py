@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-One "step" is one prefill pass of the attention layer over BASELINE config 3 (8 packed
+One "step" is one prefill pass of the attention layer over benchmark config 3 (8 packed
 sequences, lengths U[1024, 8192], 32-token blocks, Hq 16 / Hkv 8 / d 128, bf16):
 store_kvcache of the committed rows, then the staircase attention.  `value` is the
 attention's ALGORITHMIC throughput (4*d*Hq flops per visible (query, key) pair, masked

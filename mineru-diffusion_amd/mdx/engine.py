@@ -307,10 +307,12 @@ class BlockDiffusionEngine:
 
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
                  max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
-                 decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True):
+                 decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True,
+                 replay_ahead: bool = True):
         self.model = model
         self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
         self.max_model_len = max_model_len
+        self.replay_ahead = replay_ahead                   # graph decode: enqueue the next forward before the host bookkeeping
         self.masked_rows_only = masked_rows_only           # graph decode: logits for still-masked positions only
         self._graphs = {}
         self._temps = None
@@ -458,6 +460,9 @@ class BlockDiffusionEngine:
         g["dev_buf"].copy_(g["pin_buf"])
         g["result"] = torch.zeros(2, bs, S, dtype=torch.int64, device=dev)          # tokens, transfer flags
         g["result_host"] = torch.zeros(2, bs, S, dtype=torch.int64, pin_memory=True)
+        g["downloaded"] = torch.cuda.Event()
+        g["idx_host"] = torch.zeros(bs * S, dtype=torch.int64, pin_memory=True)       # rows still masked
+        g["idx_dev"] = torch.zeros(bs * S, dtype=torch.int64, device=dev)
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -498,7 +503,11 @@ class BlockDiffusionEngine:
             g["signature"] = signature
             g["x_host"] = h["ids"]                          # host copy of the device token blocks
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
-        g["graph"].replay()
+        ahead = g.pop("replayed_ahead", False)              # enqueued by the previous pass's `_download`?
+        for other in self._graphs.values():
+            other.pop("replayed_ahead", None)               # a forward enqueued ahead for another batch is void
+        if not (fresh and ahead):
+            g["graph"].replay()
         return g["hidden"], g
 
     def _temperatures(self, seqs):
@@ -535,7 +544,15 @@ class BlockDiffusionEngine:
         g["result"][0].copy_(x)
         g["result"][1].copy_(transfer)
         g["result_host"].copy_(g["result"], non_blocking=True)
-        torch.cuda.current_stream().synchronize()
+        g["downloaded"].record()
+        # The next pass's forward needs nothing from the host when no sequence of this pass is about
+        # to append its block (then lengths, slots and page tables stay, and the token block is on
+        # the device already): enqueue it now, so that the GPU runs it while the host does the
+        # bookkeeping below.  `_run_decode_graph` checks that this really was the next pass.
+        if self.replay_ahead and not any(s.is_caching for s in seqs):
+            g["graph"].replay()
+            g["replayed_ahead"] = True
+        g["downloaded"].synchronize()
         x_cpu, transfer_cpu = g["result_host"][0].clone(), g["result_host"][1].bool()
         g["x_host"] = x_cpu
         # one indexed write for all step maps: the sequences' maps are rows of one batch tensor
@@ -570,7 +587,12 @@ class BlockDiffusionEngine:
             for s in seqs:
                 s.current_denoise_step += 1
             return 0
-        idx_dev = idx.to(self.device, non_blocking=True)
+        # through pinned memory: a copy from pageable memory would hold the host until the stream,
+        # which may already hold the next forward, has drained
+        n = idx.numel()
+        g["idx_host"][:n].copy_(idx)
+        idx_dev = g["idx_dev"][:n]
+        idx_dev.copy_(g["idx_host"][:n], non_blocking=True)
         logits = F.linear(hidden.view(bs * S, -1).index_select(0, idx_dev), self.model.lm_head)
         temps = self._temperatures(seqs)
         if len(set(self._temps[0])) == 1:

@@ -168,7 +168,7 @@ def test_paged_is_invariant_to_page_placement(dev):
 
 
 def test_paged_config2_shape(dev):
-    """BASELINE config 2 shape: 16 sequences, prefix U[512, 4096] + 32, page 256 (small pool here)."""
+    """benchmark config 2 shape: 16 sequences, prefix U[512, 4096] + 32, page 256 (small pool here)."""
     g = torch.Generator().manual_seed(2)
     ctxs = [int(x) + 32 for x in torch.randint(512, 4097, (16,), generator=g)]
     _check_paged(dev, ctxs, seed=2, pool=300)

@@ -154,3 +154,27 @@ def test_masked_rows_only_sampling_matches_full_logits(dev, temps):
         same = sum(int(a == b) for a, b in zip(ta, tb))
         assert same >= 90, f"only {same}/96 tokens agree"
         assert sum(int(a == b) for a, b in zip(ma, mb)) >= 90
+
+
+def test_replay_ahead_changes_nothing(dev):
+    """Enqueuing the next decode forward before the host bookkeeping of the current pass is pure
+    scheduling: same tokens, same step maps, same pass count, with a request that arrives late
+    (its prefill runs between two decode passes) and sequences of different lengths."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for ahead in (False, True):
+        eng = BlockDiffusionEngine(model, num_pages=20, shuffle_pages_seed=4, decode_graphs=True, max_model_len=1024,
+                                   replay_ahead=ahead)
+        g = torch.Generator().manual_seed(6)
+        sp = SamplingParams(max_new_tokens=64, ignore_eos=True, transfer_count=4)
+        seqs = [eng.add_request(torch.randint(0, 900, (n,), generator=g).tolist(), sp) for n in (200, 45)]
+        for _ in range(5):
+            eng.step()
+        seqs.append(eng.add_request(torch.randint(0, 900, (77,), generator=g).tolist(),
+                                    SamplingParams(max_new_tokens=32, ignore_eos=True, transfer_count=8)))
+        eng.generate()
+        outs.append(([s.completion_token_ids for s in seqs], [list(s.step_map) for s in seqs], dict(eng.stats)))
+    (ta, ma, sa), (tb, mb, sb) = outs
+    assert ta == tb and ma == mb
+    assert sa["decode_passes"] == sb["decode_passes"] and sa["prefill_passes"] == sb["prefill_passes"] == 2

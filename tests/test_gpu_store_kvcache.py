@@ -95,7 +95,7 @@ def test_store_out_of_range_slots_are_skipped(dev):
 
 
 def test_store_full_size_round_trip(dev):
-    """BASELINE config 3 size (about 36.9k tokens): store, gather back through the slots, compare."""
+    """benchmark config 3 size (about 36.9k tokens): store, gather back through the slots, compare."""
     import mdx
     g = torch.Generator().manual_seed(33)
     N, hkv, d, page = 36864 + 17, 8, 128, 256

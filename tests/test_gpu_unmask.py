@@ -156,7 +156,7 @@ def test_unmask_block_lengths(dev):
 
 
 def test_unmask_full_size(dev):
-    """BASELINE config 4: [32 x 32 x 151936] bf16 N(0, 3^2), 50-100 % masked, k = 4, thr 0.9.
+    """benchmark config 4: [32 x 32 x 151936] bf16 N(0, 3^2), 50-100 % masked, k = 4, thr 0.9.
     The oracle runs on every 8th row's softmax in fp64; argmax is checked on all rows."""
     import mdx
     g = torch.Generator().manual_seed(4)

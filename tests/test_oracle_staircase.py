@@ -134,7 +134,7 @@ def test_paged_equals_contiguous_and_ignores_placement():
 
 
 def test_config1_anchor():
-    """BASELINE config 1: B=1, prefix 1024 + block 32, Hq 16, Hkv 8, d 128, fp32; the block's
+    """benchmark config 1: B=1, prefix 1024 + block 32, Hq 16, Hkv 8, d 128, fp32; the block's
     rows of the staircase mask are all True and the op equals unmasked SDPA; 276.8 MFLOP."""
     g = torch.Generator().manual_seed(1)
     L = 1056
