@@ -313,14 +313,18 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     *reinterpret_cast<bf16x2*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + lane * 2) = out;
 }
 
-// Keys per split: enough workgroups to fill 256 CUs a few times over, but no smaller than one page.
+// Keys per split.  Two workgroups fit on a CU, and page tables are rarely full: aiming for about 2.7
+// workgroups per CU at the table's capacity leaves, at typical fill, roughly one resident round of
+// workgroups, which is where both the 16-sequence benchmark shape and the engine's 32-sequence decode
+// pass are fastest (smaller splits add partials and combine work, larger ones an uneven tail).
+// Never smaller than one page-aligned unit of kChunkAlign keys.
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size) {
     static const int forced = [] { const char* e = getenv("MDX_PAGED_CHUNK"); return e ? atoi(e) : 0; }();
     if (forced >= kChunkAlign && forced % kChunkAlign == 0) return forced;
     const int64_t max_keys = (int64_t)max_pages * page_size;
-    const int64_t target_wgs = 1024;
+    const int64_t target_wgs = 700;
     int64_t chunk = (int64_t)bs * head_groups * max_keys / target_wgs;
-    chunk = (chunk + kChunkAlign - 1) / kChunkAlign * kChunkAlign;
+    chunk = (chunk + kChunkAlign / 2) / kChunkAlign * kChunkAlign;          // to the nearest multiple
     if (chunk < kChunkAlign) chunk = kChunkAlign;
     if (chunk > max_keys) chunk = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;
     return (int)chunk;
