@@ -21,6 +21,7 @@ import math
 import os
 import sys
 import time
+from itertools import count
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
@@ -422,8 +423,10 @@ def main():
         rows4 = 32 * S
         ws_bytes4 = L.mdx_confidence_argmax_workspace_bytes(rows4, VOCAB)
         ws4 = torch.empty(max(ws_bytes4, 16), dtype=torch.uint8, device=dev)
-        tok0 = c4["tokens"].to(dev)
-        dtok = tok0.clone()
+        # every step starts from the same masked blocks: one copy of them per call, made beforehand
+        n_calls = W + K + 10
+        dtoks = c4["tokens"].to(dev).unsqueeze(0).repeat(n_calls, 1, 1).contiguous()
+        calls = count()
         x0_4 = torch.empty(32, S, dtype=torch.int64, device=dev)
         p_4 = torch.empty(32, S, dtype=torch.float32, device=dev)
         tr_4 = torch.empty(32, S, dtype=torch.uint8, device=dev)
@@ -431,7 +434,7 @@ def main():
 
         def unmask(i):
             lg = c4["logits"][i % len(c4["logits"])]
-            dtok.copy_(tok0)                       # every step starts from the same masked block (8 KB copy)
+            dtok = dtoks[next(calls) % n_calls]
             rc = L.mdx_unmask_step(lg.data_ptr(), VOCAB, 0, None, None, 0, dtok.data_ptr(), MASK_ID, 0.9, 4,
                                    x0_4.data_ptr(), p_4.data_ptr(), tr_4.data_ptr(), cnt_4.data_ptr(), 32, S, VOCAB,
                                    ws4.data_ptr(), ws_bytes4, raw_stream())
