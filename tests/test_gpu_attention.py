@@ -167,6 +167,29 @@ def test_paged_is_invariant_to_page_placement(dev):
     assert torch.equal(o1, o2)
 
 
+def test_paged_many_sequences_and_wide_tables(dev):
+    """Launch geometries: more than 64 sequences (rectangular grid instead of the dense numbering),
+    exactly 64, and page tables much wider than the contexts need (the split size follows the
+    table width, so most splits are empty), with padding rows in between."""
+    import mdx
+    g = torch.Generator().manual_seed(21)
+    for bs in (64, 70, 130):
+        ctxs = [int(x) for x in torch.randint(1, 700, (bs,), generator=g)]
+        ctxs[3] = 0
+        ctxs[-1] = 1
+        _check_paged(dev, ctxs, seed=bs, pool=3 * bs + 8)
+    # wide table: 20 pages per row, contexts of one to three pages
+    ctxs = [300, 33, 760, 0, 512]
+    q, kc, vc, bt, lens = _paged_inputs(g, ctxs, pool=40)
+    wide = torch.full((len(ctxs), 20), -1, dtype=torch.int32)
+    wide[:, :bt.shape[1]] = bt
+    scale = 1 / math.sqrt(128)
+    o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens.to(dev),
+                                    block_table=wide.to(dev), softmax_scale=scale, causal=False)
+    ref = oracle.paged_block_attn(q, kc, vc, bt, lens, scale)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
+
+
 def test_paged_config2_shape(dev):
     """benchmark config 2 shape: 16 sequences, prefix U[512, 4096] + 32, page 256 (small pool here)."""
     g = torch.Generator().manual_seed(2)
