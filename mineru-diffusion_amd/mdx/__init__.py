@@ -11,6 +11,9 @@ reference functions they replace):
   Attention                 nanovllm/layers/sdar_attention.py:19-57
   Sampler                   nanovllm/layers/sampler.py:6-61
   Context / set_context ..  nanovllm/utils/context.py
+  rms_norm                  nanovllm/layers/layernorm.py:43-51 (RMSNorm.forward, with or without residual)
+  silu_and_mul              nanovllm/layers/activation.py:13-16 (SiluAndMul.forward)
+  qk_norm_rope_store        nanovllm/models/sdar.py:79-83 in one launch (q/k norm, rotary, KV store)
 
 Every op runs in libmdx.so; importing an op works without a GPU, calling one
 without the built library or on a non-GPU tensor raises.

@@ -11,9 +11,10 @@ kernels can be driven exactly as the engine drives them:
   decoder layer structure         nanovllm/models/sdar.py:68-181, layers/layernorm.py:16-40,
                                   layers/rotary_embedding.py:6-48, layers/embed_head.py:61-67
 
-The decoder is a random-init scaffold built from stock PyTorch ops (its GEMMs are library
-GEMMs); attention, the KV store and the unmask step go through libmdx.  There is no vision
-tower, tokenizer, weight loader or tensor parallelism here.
+The decoder is a random-init scaffold whose GEMMs are stock PyTorch (library) GEMMs; attention,
+the KV store, the norms, the activation and the unmask step go through libmdx.  Decode passes can
+replay a captured HIP graph (model_runner.py:198-259).  There is no vision tower, tokenizer,
+weight loader or tensor parallelism here.
 """
 from __future__ import annotations
 
