@@ -313,20 +313,23 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     *reinterpret_cast<bf16x2*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + lane * 2) = out;
 }
 
-// Keys per split.  Two workgroups fit on a CU, and page tables are rarely full: aiming for about 2.7
-// workgroups per CU at the table's capacity leaves, at typical fill, roughly one resident round of
-// workgroups, which is where both the 16-sequence benchmark shape and the engine's 32-sequence decode
-// pass are fastest (smaller splits add partials and combine work, larger ones an uneven tail).
-// Never smaller than one page-aligned unit of kChunkAlign keys.
+// Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
+// kernel is fastest with 1.5 to 1.8 workgroups per CU in total (just under the two per CU that are
+// resident at once: one round, no tail of late workgroups), with splits of at least 512 keys (a
+// workgroup's fixed cost is worth some 300 keys of streaming) and with no split at all once there
+// is a (sequence, head group) pair per CU (in the engine's decode pass at batch 32 that beats two
+// splits per sequence by 4 %: no partials to write and no combine launch).  The host knows the page-table width, not the lengths:
+// tables are taken to be about 65 % full, and the last split of a sequence to be half a split.
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size) {
     static const int forced = [] { const char* e = getenv("MDX_PAGED_CHUNK"); return e ? atoi(e) : 0; }();
     if (forced >= kChunkAlign && forced % kChunkAlign == 0) return forced;
     const int64_t max_keys = (int64_t)max_pages * page_size;
-    const int64_t target_wgs = 700;
-    int64_t chunk = (int64_t)bs * head_groups * max_keys / target_wgs;
-    chunk = (chunk + kChunkAlign / 2) / kChunkAlign * kChunkAlign;          // to the nearest multiple
-    if (chunk < kChunkAlign) chunk = kChunkAlign;
-    if (chunk > max_keys) chunk = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;
+    const int64_t whole = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;   // one split per sequence
+    const double per_pair = 500.0 / ((double)bs * head_groups) - 0.5;                 // workgroups per pair
+    if ((int64_t)bs * head_groups >= 256 || per_pair <= 1.0) return (int)whole;         // a pair per CU: no partials, no combine
+    int64_t chunk = (int64_t)(0.65 * (double)max_keys / per_pair / kChunkAlign + 0.5) * kChunkAlign;
+    if (chunk < 2 * kChunkAlign) chunk = 2 * kChunkAlign;
+    if (2 * chunk >= max_keys && (int64_t)bs * head_groups >= 200) chunk = whole;   // two short splits only to fill CUs
     return (int)chunk;
 }
 
