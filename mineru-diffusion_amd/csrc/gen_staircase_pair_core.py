@@ -219,15 +219,36 @@ def v_address_ops(slot_sreg):
     return ops
 
 
-def check_rescale(uid, cb):
+def mask_ops(b):
+    """S[b] value -> -inf wherever its key is not visible to this lane's query (the test of the
+    exponential's mask; applying it twice is harmless)."""
+    ops = []
+    for h in range(2):
+        for u in range(2):
+            for i in range(16):
+                r = sreg(b, h, u, i)
+                ops += [f"v_add_u32_e32 {T[i % 4]}, {key_const(u, i)}, {MREL}",
+                        f"v_cmp_lt_u32_e32 vcc, {T[i % 4]}, %[mlim]",
+                        f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc"]
+    return ops
+
+
+def check_rescale(uid, cb, masked):
     """Lazy running-max update from MX = row max of S' = c s - m: only when some query of either
     head exceeds the stale max by more than 2^8.  The rare path moves m up by delta = max(MX, 0):
     the -m tuple and the scores of tile t (computed with the old m) go down by delta, the row sums
-    and O^T (accumulation registers) are scaled by 2^-delta."""
+    and O^T (accumulation registers) are scaled by 2^-delta.
+    MX was taken over all 64 keys of the tile, visible or not: an upper bound of the visible maximum,
+    good enough to decide that nothing has to move.  When something may have to move and the tile
+    holds keys that some query must not see, the maximum is taken again over the visible keys only:
+    a hidden key with a score far above every visible one must not raise m (the visible terms, and
+    everything accumulated so far, would be scaled to zero)."""
     lab = f".Lskip_{uid}_%="
     out = [f"v_max_f32_e32 {T[0]}, {MX[0]}, {MX[1]}",
            f"v_cmp_lt_f32_e32 vcc, 0x41000000, {T[0]}",
            f"s_cbranch_vccz {lab}"]
+    if masked:
+        out += mask_ops(cb) + rowmax_ops(cb)
     for h in range(2):
         out.append(f"v_max_f32_e32 {T[0]}, 0, {MX[h]}")
         out.append(f"v_exp_f32_e64 {T[1]}, -{T[0]}")
@@ -345,6 +366,12 @@ def prologue():
     out += k_address_ops(S_R0)
     qk0_block(out)
     out.append("s_nop 15")
+    # m starts as the maximum over the keys each query may see: when the wavefront's first limit lies
+    # inside tile 0 the hidden keys are taken out first (keys before the sequence are copies of its
+    # first key, which every query sees: they cannot raise the maximum)
+    out += [f"s_movk_i32 {S_TMP}, 64", f"s_cmp_gt_i32 {S_TMP}, %[whm]", "s_cbranch_scc0 .Lplain0_%="]
+    out += mask_ops(0)
+    out.append(".Lplain0_%=:")
     out += rowmax_ops(0)
     for h in range(2):
         for i in range(16):
@@ -391,7 +418,7 @@ def body(cb, masked):
     for n in range(RING_DEPTH):
         rg.last[n] = n
     rg.issued = RING_DEPTH
-    out += check_rescale(uid, cb)
+    out += check_rescale(uid, cb, masked)
     for n in range(32):
         if n == 16:
             # tile t+2 (loaded two iterations ago; tile t+3 may still be in flight) has landed; after

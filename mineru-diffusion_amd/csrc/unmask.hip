@@ -186,10 +186,11 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
                     s *= fast_exp2((m - cm) * c);
                     m = cm;
                 }
-                const float mc = -m * c;
+                // (x - m) first, then the scale: the difference of two logits is exact, whereas
+                // x * c - m * c would carry the rounding of m * c (2^-24 |m c|) into every term
                 float acc = 0.f;
 #pragma unroll
-                for (int i = 0; i < EPC; ++i) acc += fast_exp2(fmaf(x[i], c, mc));
+                for (int i = 0; i < EPC; ++i) acc += fast_exp2((x[i] - m) * c);
                 s += acc;
             }
         }
@@ -208,10 +209,9 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
                 s *= fast_exp2((m - cm) * c);
                 m = cm;
             }
-            const float mc = -m * c;
             float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < EPC; ++i) acc += fast_exp2(fmaf(x[i], c, mc));
+            for (int i = 0; i < EPC; ++i) acc += fast_exp2((x[i] - m) * c);
             s += acc;
         }
         p.m = m;

@@ -217,3 +217,56 @@ def test_decode_matches_prefill_last_block(dev):
                                         block_table=table.to(dev), softmax_scale=1 / math.sqrt(d), causal=False)
     torch.cuda.synchronize()
     assert (o_dec[0].float() - o_pre[-32:].float()).abs().max().item() < 1e-2
+
+
+@pytest.mark.parametrize("scale_qk", [3.0, 6.0])
+def test_attention_with_peaked_scores(dev, scale_qk):
+    """Scores with a standard deviation of 9 and 36 (softmax close to one-hot, running maxima that
+    jump by hundreds between key tiles): the lazily rescaled accumulators must neither overflow nor
+    lose the terms that still matter at bf16 output precision.  The kernels (like the reference,
+    block_prefill_attention_v2.py:80,194) round q * scale * log2(e) to bf16 before the product; at
+    scores of this size that rounding alone moves the result by more than the tolerance, so the
+    queries are given here already multiplied and rounded, with softmax_scale = ln 2: the kernel's
+    own factor is then 1 and kernel and oracle start from the same numbers."""
+    import mdx
+    g = torch.Generator().manual_seed(31)
+    c = math.log2(math.e) / math.sqrt(128)
+    ln2 = math.log(2.0)
+    lens = [333, 1200]
+    q, k, v, cu = _packed(g, lens, 4, 2)
+    q, k = (q.float() * scale_qk * scale_qk * c).bfloat16(), k
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, softmax_scale=ln2)
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, 32, scale=ln2)
+    assert torch.isfinite(o).all()
+    err = (o.float().cpu() - ref).abs().max().item()
+    assert err < 1.5 * TOL, err                              # outputs are near-single V rows of magnitude up to 4
+    # the same through the paged kernel
+    gq, kc, vc, bt, ctx = _paged_inputs(g, [700, 40, 2500], hq=4, hkv=2, pool=16)
+    gq = (gq.float() * scale_qk * scale_qk * c).bfloat16()
+    od = mdx.flash_attn_with_kvcache(gq.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=ctx.to(dev), block_table=bt.to(dev),
+                                     softmax_scale=ln2, causal=False)
+    refd = oracle.paged_block_attn(gq, kc, vc, bt, ctx, ln2)
+    assert torch.isfinite(od).all()
+    err = (od.float().cpu() - refd).abs().max().item()
+    assert err < 1.5 * TOL, err
+
+
+def test_attention_with_uniformly_low_and_constant_scores(dev):
+    """All scores equal (K = 0: the output is the mean of the visible V rows) and all scores far
+    below zero (q = -k direction): nothing in the kernels may depend on the scores' absolute level."""
+    import mdx
+    g = torch.Generator().manual_seed(32)
+    lens = [200]
+    q, k, v, cu = _packed(g, lens, 2, 1)
+    k0 = torch.zeros_like(k)
+    o = mdx.sparse_attn_varlen(q.to(dev), k0.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    ref = oracle.staircase_attn_varlen(q, k0, v, cu, 32)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
+    # rows of the last block see all 200 keys: plain mean of V
+    assert (o[-1].float().cpu() - v.float().mean(0).expand(2, -1)).abs().max().item() < TOL
+    kneg = (-4.0 * q[:, :1].float()).bfloat16()             # score(i, i) = -4 |q_i|^2 / sqrt(d): about -45 on the diagonal
+    # queries already multiplied by scale * log2(e) and rounded, softmax_scale = ln 2 (see the test above)
+    qs = (q.float() * (math.log2(math.e) / math.sqrt(128))).bfloat16()
+    o = mdx.sparse_attn_varlen(qs.to(dev), kneg.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, softmax_scale=math.log(2.0))
+    ref = oracle.staircase_attn_varlen(qs, kneg, v, cu, 32, scale=math.log(2.0))
+    assert (o.float().cpu() - ref).abs().max().item() < TOL

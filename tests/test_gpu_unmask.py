@@ -14,7 +14,7 @@ def _f64(t: torch.Tensor) -> np.ndarray:
     return t.detach().cpu().to(torch.float64).numpy()
 
 
-def _check_conf(dev, logits, temps=None, noise=None):
+def _check_conf(dev, logits, temps=None, noise=None, rtol=2e-5):
     import mdx
     x0, p = mdx.confidence_argmax(logits.to(dev), None if temps is None else temps.to(dev),
                                   None if noise is None else noise.to(dev))
@@ -22,7 +22,7 @@ def _check_conf(dev, logits, temps=None, noise=None):
     ex0, ep = oracle.confidence_argmax(_f64(logits), None if temps is None else temps.numpy(),
                                        None if noise is None else noise.numpy())
     assert np.array_equal(x0.cpu().numpy(), ex0)
-    np.testing.assert_allclose(p.cpu().numpy(), ep, rtol=2e-5, atol=1e-30)
+    np.testing.assert_allclose(p.cpu().numpy(), ep, rtol=rtol, atol=1e-30)
     return x0, p
 
 
@@ -176,3 +176,23 @@ def test_unmask_full_size(dev):
     assert np.array_equal(transfer.cpu().numpy(), etr)
     assert np.array_equal(dtok.cpu().numpy(), np.where(etr, ex0.numpy(), tokens.numpy()))
     assert (count.cpu().numpy() == 4).all()
+
+
+def test_confidence_extreme_logits(dev):
+    """Large magnitudes (the bf16 range allows them), -inf entries (a masked-out vocabulary slice)
+    and a row whose maximum sits in the last, unaligned elements."""
+    g = torch.Generator().manual_seed(41)
+    logits = (torch.randn(3, 4, 5003, generator=g) * 3)
+    logits[0] *= 1000.0                                     # differences of thousands: one-hot softmax
+    logits[1, :, 100:2000] = float("-inf")
+    logits[2, 0, -1] = 50.0
+    logits[2, 1, 0] = 50.0
+    logits[2, 2, 5001] = 50.0
+    x0, p = _check_conf(dev, logits.bfloat16())
+    assert x0[2, 0].item() == 5002 and x0[2, 1].item() == 0 and x0[2, 2].item() == 5001
+    assert torch.isfinite(p).all() and (p > 0).all() and (p <= 1).all()
+    # With a temperature the reference rounds logits / T to fp32 before the softmax (sampler.py:13) and
+    # so does the oracle; at |logits / T| of 10^4..10^5 that rounding alone moves a probability by up
+    # to a percent, while the kernel scales the exact difference to the maximum: the argmax must
+    # still agree exactly, the probability within that rounding.
+    _check_conf(dev, logits.bfloat16(), temps=torch.tensor([0.05, 1.0, 7.0]), rtol=3e-2)
