@@ -219,8 +219,9 @@ def test_decode_matches_prefill_last_block(dev):
     assert (o_dec[0].float() - o_pre[-32:].float()).abs().max().item() < 1e-2
 
 
+@pytest.mark.parametrize("hq,hkv,S", [(4, 2, 32), (4, 2, 4), (3, 1, 32), (4, 2, 128)])
 @pytest.mark.parametrize("scale_qk", [3.0, 6.0])
-def test_attention_with_peaked_scores(dev, scale_qk):
+def test_attention_with_peaked_scores(dev, scale_qk, hq, hkv, S):
     """Scores with a standard deviation of 9 and 36 (softmax close to one-hot, running maxima that
     jump by hundreds between key tiles): the lazily rescaled accumulators must neither overflow nor
     lose the terms that still matter at bf16 output precision.  The kernels (like the reference,
@@ -233,15 +234,15 @@ def test_attention_with_peaked_scores(dev, scale_qk):
     c = math.log2(math.e) / math.sqrt(128)
     ln2 = math.log(2.0)
     lens = [333, 1200]
-    q, k, v, cu = _packed(g, lens, 4, 2)
+    q, k, v, cu = _packed(g, lens, hq, hkv)
     q, k = (q.float() * scale_qk * scale_qk * c).bfloat16(), k
-    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, softmax_scale=ln2)
-    ref = oracle.staircase_attn_varlen(q, k, v, cu, 32, scale=ln2)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S, softmax_scale=ln2)
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, S, scale=ln2)
     assert torch.isfinite(o).all()
     err = (o.float().cpu() - ref).abs().max().item()
     assert err < 1.5 * TOL, err                              # outputs are near-single V rows of magnitude up to 4
     # the same through the paged kernel
-    gq, kc, vc, bt, ctx = _paged_inputs(g, [700, 40, 2500], hq=4, hkv=2, pool=16)
+    gq, kc, vc, bt, ctx = _paged_inputs(g, [700, 40, 2500], hq=hq, hkv=hkv, pool=16)
     gq = (gq.float() * scale_qk * scale_qk * c).bfloat16()
     od = mdx.flash_attn_with_kvcache(gq.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=ctx.to(dev), block_table=bt.to(dev),
                                      softmax_scale=ln2, causal=False)
@@ -270,3 +271,14 @@ def test_attention_with_uniformly_low_and_constant_scores(dev):
     o = mdx.sparse_attn_varlen(qs.to(dev), kneg.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, softmax_scale=math.log(2.0))
     ref = oracle.staircase_attn_varlen(qs, kneg, v, cu, 32, scale=math.log(2.0))
     assert (o.float().cpu() - ref).abs().max().item() < TOL
+
+
+def test_prefill_many_short_sequences(dev):
+    """More than 64 sequences (rectangular launch grid instead of the dense numbering), exactly 64,
+    lengths from 0 to a few blocks, block sizes below and above the 32 rows of a wavefront."""
+    g = torch.Generator().manual_seed(51)
+    for B, S in ((150, 32), (64, 32), (90, 4), (70, 128)):
+        lens = [int(x) for x in torch.randint(0, 140, (B,), generator=g)]
+        lens[0], lens[5], lens[-1] = 1, 0, 139
+        _check_prefill(dev, lens, S, hq=4, hkv=2, seed=B + S)
+        _check_prefill(dev, lens[:7], S, hq=3, hkv=1, seed=B)          # odd head ratio: the one-head kernel
