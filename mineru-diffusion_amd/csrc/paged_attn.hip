@@ -35,6 +35,12 @@ constexpr int kMaxSq = 32;
 constexpr int kThreads = 256;      // 4 wavefronts, 2 workgroups per CU
 constexpr int kChunkAlign = 256;   // split boundaries are multiples of this many keys
 
+__device__ __forceinline__ int wave_sum(int x) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o);
+    return __builtin_amdgcn_readfirstlane(x);      // the same in every lane: say so to the compiler
+}
+
 struct PagedParams {
     const __bf16* q; __bf16* o; const __bf16* k_cache; const __bf16* v_cache;
     int64_t q_sb, q_ss, q_sh, o_sb, o_ss, o_sh;     // element strides
@@ -47,6 +53,12 @@ struct PagedParams {
     int num_q_heads;
     float c;                                        // scale * log2(e)
     float* part_o; float* part_ml;                  // [bs, Hq, nsplit, 32, 128] and [bs, Hq, nsplit, 2, 32]
+    // non-null: the attention kernel picks the split size (>= chunk) from the lengths and leaves it
+    // here for the combine kernel.  A float on purpose: an int store in the attention kernel could
+    // alias the int page table and lengths for the compiler, which would then stop fetching those
+    // through the scalar cache and wait on the vector-memory counter for them, draining the K/V
+    // prefetch queue (measured: 78 -> 120 us).  Split sizes are far below 2^24, so the value is exact.
+    float* span_out;
 };
 
 template <int HPW, int DEPTH>
@@ -66,10 +78,22 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
     const int head = hg * HPW + wave / KW;          // and query head
 
     // ---- workgroup -> (sequence b, split) ------------------------------------------------------
-    int b, split;
+    int b, split, span = P.chunk;
     if (P.bs <= 64) {
+        const int ctx_l = lane < P.bs ? max(0, P.context_lens[lane]) : 0;
+        if (P.span_out) {
+            // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
+            // nothing to combine) -- unless one of them is much longer than the rest and would keep
+            // its CU busy long after the others are done.  Only the device knows the lengths: the
+            // split grows from the host's size to 1.25 x the mean length, so that only sequences
+            // well above the mean are cut, into pieces of about the mean.
+            const int live = wave_sum(ctx_l > 0 ? 1 : 0);
+            const int mean = wave_sum(ctx_l) / max(live, 1);
+            span = max(span, (mean + mean / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
+            if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
+        }
         int n = 0;                                  // splits of sequence `lane` (padding rows get one)
-        if (lane < P.bs) n = max(1, (P.context_lens[lane] + P.chunk - 1) / P.chunk);
+        if (lane < P.bs) n = max(1, (ctx_l + span - 1) / span);
         int before = 0;
         for (int s = 0; s < P.bs; ++s) {
             const int ns = __builtin_amdgcn_readlane(n, s);
@@ -84,9 +108,8 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         b = blockIdx.y / P.nsplit;
         split = blockIdx.y % P.nsplit;
     }
-
     const int ctx = P.context_lens[b];
-    const int n_valid_splits = (ctx + P.chunk - 1) / P.chunk;
+    const int n_valid_splits = (ctx + span - 1) / span;
     if (ctx <= 0) {
         // graph-padding row: defined output (zeros), written by its split 0
         if (split == 0) {
@@ -97,9 +120,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         }
         return;
     }
-    const int key_begin = split * P.chunk;
+    const int key_begin = split * span;
     if (key_begin >= ctx) return;
-    const int key_end = min(ctx, key_begin + P.chunk);
+    const int key_end = min(ctx, key_begin + span);
     const int kvh = (hg * HPW) / P.heads_per_kv;
 
     const bool row_ok = r < P.sq;
@@ -274,7 +297,8 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     const int b = (int)(row / P.sq / P.num_q_heads);
     const int ctx = P.context_lens[b];
     const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
-    const int nv = (ctx + P.chunk - 1) / P.chunk;
+    const int span = P.span_out ? (int)*P.span_out : P.chunk; // the attention kernel's choice
+    const int nv = (ctx + span - 1) / span;
     if (nv <= 1) return;                                   // written directly by the attention kernel
     // The kernel is a chain of memory latencies, not of bytes: every load of a group of four
     // splits is issued before the first value is used.
@@ -316,17 +340,25 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
 // kernel is fastest with 1.5 to 1.8 workgroups per CU in total (just under the two per CU that are
 // resident at once: one round, no tail of late workgroups), with splits of at least 512 keys (a
-// workgroup's fixed cost is worth some 300 keys of streaming) and with no split at all once there
+// workgroup's fixed cost is worth some 300 keys of streaming) and with whole sequences once there
 // is a (sequence, head group) pair per CU (in the engine's decode pass at batch 32 that beats two
-// splits per sequence by 4 %: no partials to write and no combine launch).  The host knows the page-table width, not the lengths:
-// tables are taken to be about 65 % full, and the last split of a sequence to be half a split.
-int pick_chunk(int bs, int head_groups, int max_pages, int page_size) {
+// splits per sequence by 4 %: no partials to write, nothing to combine).  The host knows the
+// page-table width, not the lengths: tables are taken to be about 65 % full, and the last split of
+// a sequence to be half a split.  In the pair-per-CU case the grid allows two splits per sequence
+// and the kernel itself, which sees the lengths, cuts only sequences well above the mean
+// (*device_span; the dense workgroup numbering that this needs exists for up to 64 sequences).
+int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* device_span) {
     static const int forced = [] { const char* e = getenv("MDX_PAGED_CHUNK"); return e ? atoi(e) : 0; }();
+    *device_span = false;
     if (forced >= kChunkAlign && forced % kChunkAlign == 0) return forced;
     const int64_t max_keys = (int64_t)max_pages * page_size;
     const int64_t whole = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;   // one split per sequence
     const double per_pair = 500.0 / ((double)bs * head_groups) - 0.5;                 // workgroups per pair
-    if ((int64_t)bs * head_groups >= 256 || per_pair <= 1.0) return (int)whole;         // a pair per CU: no partials, no combine
+    if ((int64_t)bs * head_groups >= 256 || per_pair <= 1.0) {
+        if (bs > 64 || whole < 4 * kChunkAlign) return (int)whole;
+        *device_span = true;
+        return (int)((whole / 2 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
+    }
     int64_t chunk = (int64_t)(0.65 * (double)max_keys / per_pair / kChunkAlign + 0.5) * kChunkAlign;
     if (chunk < 2 * kChunkAlign) chunk = 2 * kChunkAlign;
     if (2 * chunk >= max_keys && (int64_t)bs * head_groups >= 200) chunk = whole;   // two short splits only to fill CUs
@@ -347,10 +379,11 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
     if (bs <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pages <= 0 || page_size <= 0) return 0;
     const int G = num_q_heads / num_kv_heads;
     const int HPW = (G % 2 == 0) ? 2 : 1;
-    const int chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size);
+    bool device_span;
+    const int chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size, &device_span);
     const int nsplit = nsplit_of(max_pages, page_size, chunk);
     if (nsplit <= 1) return 0;
-    return (int64_t)bs * num_q_heads * nsplit * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float);
+    return (int64_t)bs * num_q_heads * nsplit * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;   // + the split size
 }
 
 extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void* v_cache,
@@ -394,19 +427,21 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     P.bs = bs; P.sq = sq; P.heads_per_kv = G; P.page_size = page_size; P.max_pages = max_pages;
     P.page_shift = -1;
     for (int i = 0; i < 31; ++i) if (page_size == (1 << i)) P.page_shift = i; P.num_pages = num_pages;
-    P.chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size);
+    bool device_span;
+    P.chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size, &device_span);
     P.nsplit = nsplit_of(max_pages, page_size, P.chunk);
     P.num_q_heads = num_q_heads;
     P.c = scale * kLog2e;
-    P.part_o = nullptr; P.part_ml = nullptr;
+    P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr;
     if (P.nsplit > 1) {
         const int64_t n_slots = (int64_t)bs * num_q_heads * P.nsplit;
-        const int64_t need = n_slots * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float);
+        const int64_t need = n_slots * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;
         MDX_REQUIRE(workspace && workspace_bytes >= need, MDX_EWORKSPACE,
                     "paged_block_attn: workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
         MDX_REQUIRE(mdx::aligned16(workspace), MDX_EWORKSPACE, "paged_block_attn: workspace not 16-byte aligned");
         P.part_o = static_cast<float*>(workspace);
         P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
+        if (device_span) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
     }
     // head group fastest, then the dense (sequence, split) index
     MDX_REQUIRE((int64_t)bs * P.nsplit <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: bs * splits %lld > 65535", (long long)bs * P.nsplit);

@@ -282,3 +282,15 @@ def test_prefill_many_short_sequences(dev):
         lens[0], lens[5], lens[-1] = 1, 0, 139
         _check_prefill(dev, lens, S, hq=4, hkv=2, seed=B + S)
         _check_prefill(dev, lens[:7], S, hq=3, hkv=1, seed=B)          # odd head ratio: the one-head kernel
+
+
+def test_paged_pair_per_cu_batches(dev):
+    """32 and more sequences of 8 KV heads: sequences stay whole unless one is far above the mean
+    length, which the kernel itself finds out and cuts (a mix of cut and whole sequences, padding
+    rows, and a batch of equal lengths where nothing is cut)."""
+    g = torch.Generator().manual_seed(61)
+    ctxs = [int(x) for x in torch.randint(200, 420, (32,), generator=g)]
+    ctxs[7], ctxs[20], ctxs[3], ctxs[31] = 3900, 1800, 0, 1
+    _check_paged(dev, ctxs, seed=61, pool=80)
+    _check_paged(dev, [777] * 40, seed=62, pool=170)
+    _check_paged(dev, [2048] * 32 + [0] * 8, seed=63, pool=270)
