@@ -344,7 +344,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // is a (sequence, head group) pair per CU (in the engine's decode pass at batch 32 that beats two
 // splits per sequence by 4 %: no partials to write, nothing to combine).  The host knows the
 // page-table width, not the lengths: tables are taken to be about 65 % full, and the last split of
-// a sequence to be half a split.  In the pair-per-CU case the grid allows two splits per sequence
+// a sequence to be half a split.  In the pair-per-CU case up to four splits per sequence are allowed
 // and the kernel itself, which sees the lengths, cuts only sequences well above the mean
 // (*device_span; the dense workgroup numbering that this needs exists for up to 64 sequences).
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* device_span) {
@@ -357,7 +357,7 @@ int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* devi
     if ((int64_t)bs * head_groups >= 256 || per_pair <= 1.0) {
         if (bs > 64 || whole < 4 * kChunkAlign) return (int)whole;
         *device_span = true;
-        return (int)((whole / 2 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
+        return (int)((whole / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
     }
     int64_t chunk = (int64_t)(0.65 * (double)max_keys / per_pair / kChunkAlign + 0.5) * kChunkAlign;
     if (chunk < 2 * kChunkAlign) chunk = 2 * kChunkAlign;
@@ -445,7 +445,10 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     }
     // head group fastest, then the dense (sequence, split) index
     MDX_REQUIRE((int64_t)bs * P.nsplit <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: bs * splits %lld > 65535", (long long)bs * P.nsplit);
-    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)(bs * P.nsplit));
+    // With device-chosen splits of at least 1.25 x the mean length, sum_b ceil(len_b / split) <= 1.8 bs:
+    // the dense numbering never needs more than 2 bs (sequence, split) pairs, whatever nsplit allows.
+    const int pairs_y = device_span ? (bs * P.nsplit < 2 * bs ? bs * P.nsplit : 2 * bs) : bs * P.nsplit;
+    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)pairs_y);
     if (HPW == 2) paged_block_attn_kernel<2, 2><<<grid, kThreads, 0, stream>>>(P);
     else          paged_block_attn_kernel<1, 1><<<grid, kThreads, 0, stream>>>(P);
     int rc = mdx::check_launch("paged_block_attn");
