@@ -285,56 +285,69 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
     }
 }
 
-// One wavefront per (sequence, head, query): merges the split partials.
+// One workgroup per (sequence, head): merges the split partials of its 32 queries; thread t takes
+// 16 consecutive d values of query t / 8.  A sequence that was not split leaves after one load, and
+// there are only bs * Hq workgroups to launch, which is what the common case costs when the
+// attention kernel decided that nothing had to be cut.  The kernel is a chain of memory latencies
+// (length -> partials -> output), not of bytes: the loads of four splits are issued together.
 __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t n_rows = (int64_t)P.bs * P.num_q_heads * P.sq;
-    if (row >= n_rows) return;
-    const int s = (int)(row % P.sq);
-    const int hq = (int)((row / P.sq) % P.num_q_heads);
-    const int b = (int)(row / P.sq / P.num_q_heads);
+    const int hq = blockIdx.x % P.num_q_heads, b = blockIdx.x / P.num_q_heads;
     const int ctx = P.context_lens[b];
-    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
     const int span = P.span_out ? (int)*P.span_out : P.chunk; // the attention kernel's choice
     const int nv = (ctx + span - 1) / span;
     if (nv <= 1) return;                                   // written directly by the attention kernel
-    // The kernel is a chain of memory latencies, not of bytes: every load of a group of four
-    // splits is issued before the first value is used.
+    const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
+    if (s >= P.sq) return;
+    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
     float M = kMinusBig, Lsum = 0.f;
-    float2 acc = make_float2(0.f, 0.f);
+    float acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
     for (int i0 = 0; i0 < nv; i0 += 4) {
         float m[4], l[4];
-        float2 po[4];
+        float4 po[4][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int64_t slot = slot0 + min(i0 + i, nv - 1);
             m[i] = P.part_ml[(slot * 2 + 0) * kMaxSq + s];
             l[i] = P.part_ml[(slot * 2 + 1) * kMaxSq + s];
-            po[i] = *reinterpret_cast<const float2*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + lane * 2);
+            const float4* src = reinterpret_cast<const float4*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) po[i][k] = src[k];
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
         const float Mn = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), M);
         const float keep = __builtin_amdgcn_exp2f(M - Mn);
-        Lsum *= keep; acc.x *= keep; acc.y *= keep;
+        Lsum *= keep;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] *= keep;
         M = Mn;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const bool on = i0 + i < nv;
             const float w = on ? __builtin_amdgcn_exp2f(m[i] - M) : 0.f;
             Lsum += on ? w * l[i] : 0.f;
-            acc.x += on ? w * po[i].x : 0.f;
-            acc.y += on ? w * po[i].y : 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                acc[4 * k + 0] += on ? w * po[i][k].x : 0.f;
+                acc[4 * k + 1] += on ? w * po[i][k].y : 0.f;
+                acc[4 * k + 2] += on ? w * po[i][k].z : 0.f;
+                acc[4 * k + 3] += on ? w * po[i][k].w : 0.f;
+            }
         }
     }
     const float inv = 1.0f / Lsum;
-    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-    bf16x2 out;
-    out[0] = (__bf16)(acc.x * inv);
-    out[1] = (__bf16)(acc.y * inv);
-    *reinterpret_cast<bf16x2*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + lane * 2) = out;
+    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+    __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        bf16x8_t out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (__bf16)(acc[8 * h + e] * inv);
+        *reinterpret_cast<bf16x8_t*>(dst + 8 * h) = out;
+    }
 }
 
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
@@ -453,7 +466,6 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     else          paged_block_attn_kernel<1, 1><<<grid, kThreads, 0, stream>>>(P);
     int rc = mdx::check_launch("paged_block_attn");
     if (rc != MDX_OK || P.nsplit == 1) return rc;
-    const int64_t n_rows = (int64_t)bs * num_q_heads * sq;
-    paged_combine_kernel<<<(unsigned)((n_rows + 3) / 4), 256, 0, stream>>>(P);
+    paged_combine_kernel<<<(unsigned)(bs * num_q_heads), 256, 0, stream>>>(P);
     return mdx::check_launch("paged_combine");
 }
