@@ -7,9 +7,11 @@
 //
 // The op is HBM-bound (each K/V byte is used by only Sq * Hq/Hkv = 64 query
 // rows), so the design goal is to keep the whole chip streaming pages:
-//  * split-KV: a workgroup owns `chunk` consecutive keys of one sequence for
-//    one group of query heads; there are far more workgroups than the bs*Hkv
-//    (sequence, KV head) pairs.  Workgroups are numbered densely over the
+//  * split-KV: a workgroup owns one split of consecutive keys of one sequence
+//    for one group of query heads; the split size is chosen so that there are
+//    1.5 to 1.8 workgroups per CU (pick_chunk), and with a (sequence, KV head)
+//    pair per CU sequences stay whole unless the kernel finds one far longer
+//    than the mean.  Workgroups are numbered densely over the
 //    (sequence, split) pairs that exist (lane b of each wavefront holds the
 //    split count of sequence b), so the launch order has no holes: the
 //    dispatcher deals consecutive workgroups round-robin to XCDs and shader
