@@ -477,32 +477,45 @@ class BlockDiffusionEngine:
         torch.cuda.synchronize()
         return g
 
+    def _graph_batch(self, bs: int) -> int:
+        """The captured batch size that serves `bs` sequences: 1, 2, 4, 8, then multiples of 16
+        (model_runner.py:233,200); the rows in excess are padding (slot -1, context length 0)."""
+        for b in (1, 2, 4, 8):
+            if bs <= b:
+                return b
+        return (bs + 15) // 16 * 16
+
     def _run_decode_graph(self, seqs):
         """Uploads the pass inputs (one copy) and replays the graph.  Within a denoising block
         nothing has to be uploaded at all: lengths, slots and page tables are those of the previous
         pass, and the token block on the device is the one the unmask step just updated in place
         (the host rows handed to the sequences by `sample` are a download of exactly that buffer)."""
         S, bs = self.c.block_size, len(seqs)
-        g = self._graphs.get(bs)
+        gbs = self._graph_batch(bs)
+        g = self._graphs.get(gbs)
         if g is None:
-            g = self._graphs[bs] = self._capture_decode(bs)
+            g = self._graphs[gbs] = self._capture_decode(gbs)
         signature = [(s.seq_id, s.num_tokens, len(s.block_table)) for s in seqs]
         rows = g.get("rows")
         fresh = (g.get("signature") == signature and rows is not None
                  and all(s.current_denoising_block is r for s, r in zip(seqs, rows)))
         if not fresh:
             h = g["host"]
-            torch.stack([s.current_denoising_block for s in seqs], out=h["ids"])
+            torch.stack([s.current_denoising_block for s in seqs], out=h["ids"][:bs])
             lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
-            torch.add(lens.unsqueeze(1), torch.arange(S), out=h["pos"])
-            h["slots"].copy_(torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32))
-            h["lens"].copy_(lens + S)
+            torch.add(lens.unsqueeze(1), torch.arange(S), out=h["pos"][:bs])
+            h["slots"].fill_(-1)                            # padding rows: nothing stored, no context (model_runner.py:203-206)
+            h["slots"][:bs] = torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32)
+            h["lens"].zero_()
+            h["lens"][:bs] = lens + S
+            h["ids"][bs:] = 0
+            h["pos"][bs:] = 0
             h["bt"].fill_(-1)
             for i, s in enumerate(seqs):
                 h["bt"][i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
             g["dev_buf"].copy_(g["pin_buf"], non_blocking=True)
             g["signature"] = signature
-            g["x_host"] = h["ids"]                          # host copy of the device token blocks
+            g["x_host"] = h["ids"][:bs]                     # host copy of the device token blocks
         set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
         ahead = g.pop("replayed_ahead", False)              # enqueued by the previous pass's `_download`?
         for other in self._graphs.values():
@@ -525,7 +538,7 @@ class BlockDiffusionEngine:
         if sp.denoising_strategy != "low_confidence_dynamic":
             raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
         if g is not None:
-            x = g["ids"]
+            x = g["ids"][:len(seqs)]
         else:
             x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
         _, _, transfer, _n = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
@@ -542,8 +555,9 @@ class BlockDiffusionEngine:
     def _download(self, seqs, g, x, transfer) -> int:
         """One download of (tokens, transfer flags) through the pinned buffer, then the per-sequence
         bookkeeping of sampler.py:56-59 as batch operations."""
-        g["result"][0].copy_(x)
-        g["result"][1].copy_(transfer)
+        bs = len(seqs)
+        g["result"][0, :bs].copy_(x)
+        g["result"][1, :bs].copy_(transfer)
         g["result_host"].copy_(g["result"], non_blocking=True)
         g["downloaded"].record()
         # The next pass's forward needs nothing from the host when no sequence of this pass is about
@@ -554,7 +568,7 @@ class BlockDiffusionEngine:
             g["graph"].replay()
             g["replayed_ahead"] = True
         g["downloaded"].synchronize()
-        x_cpu, transfer_cpu = g["result_host"][0].clone(), g["result_host"][1].bool()
+        x_cpu, transfer_cpu = g["result_host"][0, :bs].clone(), g["result_host"][1, :bs].bool()
         g["x_host"] = x_cpu
         # one indexed write for all step maps: the sequences' maps are rows of one batch tensor
         maps, map_rows = g.get("maps"), g.get("map_rows")
@@ -583,7 +597,7 @@ class BlockDiffusionEngine:
         if sp.denoising_strategy != "low_confidence_dynamic":
             raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
         S, bs, mask_id = self.c.block_size, len(seqs), seqs[0].mask_token_id
-        idx = (g["x_host"].view(-1) == mask_id).nonzero().squeeze(1)
+        idx = (g["x_host"].reshape(-1) == mask_id).nonzero().squeeze(1)
         if idx.numel() == 0:
             for s in seqs:
                 s.current_denoise_step += 1
@@ -594,7 +608,7 @@ class BlockDiffusionEngine:
         g["idx_host"][:n].copy_(idx)
         idx_dev = g["idx_dev"][:n]
         idx_dev.copy_(g["idx_host"][:n], non_blocking=True)
-        logits = F.linear(hidden.view(bs * S, -1).index_select(0, idx_dev), self.model.lm_head)
+        logits = F.linear(hidden.flatten(0, 1).index_select(0, idx_dev), self.model.lm_head)   # rows of the first bs sequences
         temps = self._temperatures(seqs)
         if len(set(self._temps[0])) == 1:
             temps = temps[:1]
@@ -602,13 +616,13 @@ class BlockDiffusionEngine:
             temps = temps.index_select(0, idx_dev // S)
         x0_rows, p_rows = confidence_argmax(logits, temps)
         if "x0" not in g:
-            g["x0"] = torch.zeros(bs * S, dtype=torch.int64, device=self.device)
-            g["x0_p"] = torch.zeros(bs * S, dtype=torch.float32, device=self.device)
+            g["x0"] = torch.zeros(g["ids"].numel(), dtype=torch.int64, device=self.device)
+            g["x0_p"] = torch.zeros(g["ids"].numel(), dtype=torch.float32, device=self.device)
         g["x0"].index_copy_(0, idx_dev, x0_rows)
         g["x0_p"].index_copy_(0, idx_dev, p_rows)
-        transfer, _n = select_transfer(g["x0"].view(bs, S), g["x0_p"].view(bs, S), g["ids"], mask_id,
+        transfer, _n = select_transfer(g["x0"][:bs * S].view(bs, S), g["x0_p"][:bs * S].view(bs, S), g["ids"][:bs], mask_id,
                                        sp.dynamic_threshold, sp.transfer_count)
-        return self._download(seqs, g, g["ids"], transfer)
+        return self._download(seqs, g, g["ids"][:bs], transfer)
 
     @torch.inference_mode()
     def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
@@ -622,7 +636,7 @@ class BlockDiffusionEngine:
             n = self._sample_masked_rows(hidden, seqs, g)
             reset_context()
             return n
-        logits = self.model.compute_logits(hidden)
+        logits = self.model.compute_logits(hidden if g is None else hidden[:len(seqs)])
         if is_prefill:
             logits = logits.view(len(seqs), self.c.block_size, -1)
         if self.on_logits is not None:

@@ -102,12 +102,15 @@ def test_decode_graph_replays_match_eager(dev):
             s.current_denoising_block = blk
         hidden = eng._run_decode_graph(seqs)[0].clone()
         torch.cuda.synchronize()
-        ids, pos = eng.prepare_decode(seqs)                # eager, its own context tensors
-        gr = eng._graphs[len(seqs)]
+        ids, pos = eng.prepare_decode(seqs)                # eager, its own tensors for the three sequences
+        gr = eng._graphs[4]                                # three sequences run in the graph captured for four
+        assert torch.equal(gr["ids"][:3], ids) and torch.equal(gr["pos"][:3], pos)
+        assert gr["lens"][3].item() == 0 and (gr["slots"][3] == -1).all()      # the padding row
         set_context(False, slot_mapping=gr["slots"], context_lens=gr["lens"], block_tables=gr["bt"], block_size=32)
-        ref = model(model.embed(ids), pos)                 # same launch geometry as the capture
+        ref = model(model.embed(gr["ids"].clone()), gr["pos"].clone())          # same launch geometry as the capture
         torch.cuda.synchronize()
         assert torch.equal(hidden, ref), f"replay {rep}: max diff {(hidden.float() - ref.float()).abs().max().item()}"
+        assert hidden[3].abs().sum().item() == hidden[3].abs().sum().item()     # padding row: finite
         if rep == 2:                                       # sequences grow between replays
             for s in seqs:
                 s.current_denoising_block = torch.randint(0, 900, (32,), generator=g)
@@ -176,5 +179,6 @@ def test_replay_ahead_changes_nothing(dev):
         eng.generate()
         outs.append(([s.completion_token_ids for s in seqs], [list(s.step_map) for s in seqs], dict(eng.stats)))
     (ta, ma, sa), (tb, mb, sb) = outs
+    assert set(eng._graphs) <= {1, 2, 4}                   # batches of 3, 2, 1 run in the graphs for 4, 2, 1
     assert ta == tb and ma == mb
     assert sa["decode_passes"] == sb["decode_passes"] and sa["prefill_passes"] == sb["prefill_passes"] == 2
