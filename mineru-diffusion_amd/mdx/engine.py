@@ -358,13 +358,29 @@ class BlockDiffusionEngine:
             scheduled.append(seq)
         if scheduled:
             return scheduled, True
-        for seq in list(self.running)[: self.max_num_seqs]:
-            if not self.block_manager.can_append(seq):
-                raise RuntimeError("KV pool exhausted (preemption is not part of this scaffold)")
-            self.block_manager.may_append(seq)
-            scheduled.append(seq)
-        assert scheduled
+        # decode (scheduler.py:44-58): a sequence that cannot get the page its next block needs makes
+        # room by preempting the sequence at the back of the queue (or itself, when it is alone)
+        while self.running and len(scheduled) < self.max_num_seqs:
+            seq = self.running.popleft()
+            while not self.block_manager.can_append(seq):
+                if self.running:
+                    self.preempt(self.running.pop())
+                else:
+                    self.preempt(seq)
+                    break
+            else:
+                self.block_manager.may_append(seq)
+                scheduled.append(seq)
+        if not scheduled:
+            raise RuntimeError("KV pool too small for a single sequence")
+        self.running.extendleft(reversed(scheduled))
         return scheduled, False
+
+    def preempt(self, seq):                                # scheduler.py:60-63: back to the queue, its pages freed;
+        seq.status = SequenceStatus.WAITING                # the next prefill recomputes its cache (the block in
+        self.block_manager.deallocate(seq)                 # progress keeps the tokens it has committed so far)
+        self.waiting.appendleft(seq)
+        self.stats["preemptions"] = self.stats.get("preemptions", 0) + 1
 
     def postprocess(self, seqs):                           # scheduler.py:65-82
         for seq in seqs:

@@ -130,3 +130,21 @@ def test_stop_token_finishes_a_sequence():
     s = eng.add_request(list(range(5)), SamplingParams(max_new_tokens=320, stop_token_ids=[10 + 7], transfer_count=4))
     eng.generate()
     assert s.num_completion_tokens == 32 and s.status == SequenceStatus.FINISHED
+
+
+def test_preemption_when_the_page_pool_runs_out():
+    """scheduler.py:44-63: with too few pages for both sequences to grow, the one at the back of the
+    queue is preempted (pages freed, back to the waiting queue), prefilled again later with the
+    tokens it has committed so far, and both still finish with the right tokens."""
+    model = ScriptedModel()
+    eng = BlockDiffusionEngine(model, num_pages=4, unmask=oracle_unmask)
+    sp = SamplingParams(max_new_tokens=288, ignore_eos=True, transfer_count=8)
+    s1 = eng.add_request(list(range(300)), sp)              # grows from 2 to 3 pages
+    s2 = eng.add_request(list(range(40)), sp)               # grows from 1 to 2 pages: 5 > 4 in total
+    eng.generate()
+    assert eng.stats["preemptions"] >= 1
+    assert sum(c["prefill"] for c in model.calls) >= 2      # the preempted sequence was prefilled again
+    for s in (s1, s2):
+        assert s.status == SequenceStatus.FINISHED and s.num_completion_tokens == 288
+        assert s.completion_token_ids == [10 + p for p in range(32)] * 9
+    assert len(eng.block_manager.free) == 4 and not eng.running and not eng.waiting
