@@ -243,6 +243,63 @@ def cpu_baseline(host3):
                 ms=round(t * 1e3, 2))
 
 
+def cpu_decode_pass(layers=2, batch=32, ctx=2112):
+    """One decode pass of the config-5 decoder on the host cores, at reduced depth: `layers` decoder
+    layers (of 28) on `batch` x 32 tokens against a cached context of `ctx` keys per sequence, plus the
+    vocabulary projection and the unmask arithmetic, fp32, stock torch CPU ops (a port of the pass,
+    not the reference's code).  Returns the pass time extrapolated to 28 layers and the committed
+    tokens/s it implies at 8 denoising passes + 1 caching pass per 32-token block."""
+    import torch.nn.functional as F
+    import oracle
+    g = torch.Generator().manual_seed(55)
+    H, I, V = 2048, 6144, VOCAB
+    rows = batch * S
+    w = dict(qkv=torch.randn((HQ + 2 * HKV) * D, H, generator=g) * 0.02, o=torch.randn(H, HQ * D, generator=g) * 0.02,
+             gu=torch.randn(2 * I, H, generator=g) * 0.02, down=torch.randn(H, I, generator=g) * 0.02, norm=torch.ones(H), hn=torch.ones(D))
+    head = torch.randn(V, H, generator=g) * 0.02
+    kc = torch.randn(batch, HKV, ctx, D, generator=g)
+    vc = torch.randn(batch, HKV, ctx, D, generator=g)
+    cos, sin = torch.ones(rows, 1, D // 2), torch.zeros(rows, 1, D // 2)
+    x = torch.randn(rows, H, generator=g)
+
+    def layer(x, res):
+        res = x + res
+        h = F.rms_norm(res, (H,), w["norm"], 1e-6)
+        qkv = h @ w["qkv"].T
+        q, k, v = qkv.split([HQ * D, HKV * D, HKV * D], -1)
+        q = oracle.rope_ref(oracle.rms_norm_ref(q.reshape(rows, HQ, D), w["hn"], 1e-6), cos, sin)
+        k = oracle.rope_ref(oracle.rms_norm_ref(k.reshape(rows, HKV, D), w["hn"], 1e-6), cos, sin)
+        kc[:, :, -S:] = k.reshape(batch, S, HKV, D).transpose(1, 2)          # the block's K/V go into the cache
+        vc[:, :, -S:] = v.reshape(batch, S, HKV, D).transpose(1, 2)
+        o = F.scaled_dot_product_attention(q.reshape(batch, S, HQ, D).transpose(1, 2), kc, vc, enable_gqa=True)
+        x = o.transpose(1, 2).reshape(rows, HQ * D) @ w["o"].T
+        res = x + res
+        h = F.rms_norm(res, (H,), w["norm"], 1e-6)
+        gate, up = (h @ w["gu"].T).chunk(2, -1)
+        return (F.silu(gate) * up) @ w["down"].T, res
+
+    def run(n_layers):
+        t0 = time.perf_counter()
+        h, res = x, torch.zeros_like(x)
+        for _ in range(n_layers):
+            h, res = layer(h, res)
+        t_layers = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        logits = F.rms_norm(h + res, (H,), w["norm"], 1e-6) @ head.T
+        p = torch.softmax(logits, -1)
+        x0 = logits.argmax(-1)
+        conf = p.gather(-1, x0[:, None])
+        t_head = time.perf_counter() - t0
+        return t_layers, t_head, float(conf.sum())
+
+    run(1)                                                                    # warm-up
+    t_layers, t_head, _ = run(layers)
+    t_pass = t_layers / layers * 28 + t_head
+    return dict(seconds_per_pass_28_layers=round(t_pass, 3), tokens_per_s=round(batch * S / 9 / t_pass, 1), cores=torch.get_num_threads(),
+                sample=f"{layers} of 28 decoder layers ({t_layers:.2f} s) extrapolated + vocabulary projection and softmax/argmax ({t_head:.2f} s), "
+                       f"batch {batch} x {S} tokens, cached context {ctx} keys, fp32 torch CPU ops; 8 denoising + 1 caching pass per block")
+
+
 def cpu_side_ops(host3, cfg4_tokens):
     """Bounded CPU timings of the two bandwidth ops, reported next to their GPU numbers."""
     import oracle
@@ -472,6 +529,8 @@ def main():
         cpu = cpu_baseline(host3)
         try:
             cpu["other_ops"] = cpu_side_ops(host3, cfg4_tokens)
+            if decode is not None:
+                cpu["other_ops"]["decode"] = cpu_decode_pass()
         except Exception as e:  # the side numbers are informative only
             cpu["other_ops"] = {"error": str(e)}
 
