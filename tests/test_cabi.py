@@ -93,3 +93,13 @@ def test_context_mirror():
     assert mdx.get_context().is_prefill and mdx.get_context().max_seqlen_q == 5
     mdx.reset_context()
     assert not mdx.get_context().is_prefill and mdx.get_context().slot_mapping is None
+
+
+def test_generated_kernel_core_is_current():
+    """staircase_pair_core.inc is the committed output of its generator: regenerate and compare."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    csrc = Path(__file__).resolve().parents[1] / "mineru-diffusion_amd" / "csrc"
+    out = subprocess.run([sys.executable, str(csrc / "gen_staircase_pair_core.py")], capture_output=True, text=True, check=True)
+    assert out.stdout == (csrc / "staircase_pair_core.inc").read_text()
