@@ -106,8 +106,10 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * sequence b sees keys 0..context_lens[b]-1 (non-causal).  Rows with
  * context_lens[b] == 0 (graph padding, model_runner.py:205-208) produce
  * zeros.  Page ids outside [0, num_pages) are treated as holding no keys.
- * The workspace holds the split-KV partial results; its size comes from
- * mdx_paged_block_attn_workspace_bytes with the same shape arguments.
+ * The workspace holds the split-KV partial results (and the split size when the
+ * kernel picks it from the lengths); its size comes from
+ * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
+ * contents need no initialisation.
  * Supported: d == 128, Sq*(Hq/Hkv) <= 64, page_size % 32 == 0, MDX_BF16.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
