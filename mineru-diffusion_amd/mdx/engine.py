@@ -309,10 +309,13 @@ class BlockDiffusionEngine:
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
                  max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
                  decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True,
-                 replay_ahead: bool = True):
+                 replay_ahead: bool = True, gumbel_seed: int | None = None):
         self.model = model
         self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
         self.max_model_len = max_model_len
+        # Gumbel noise on the scaled logits before the argmax, as Sampler.prepare draws it (sampler.py:15-18);
+        # None = plain argmax (reproducible), an int seeds a device generator (reproducible per seed)
+        self.gumbel = None if gumbel_seed is None else torch.Generator(device=model.lm_head.device).manual_seed(gumbel_seed)
         self.replay_ahead = replay_ahead                   # graph decode: enqueue the next forward before the host bookkeeping
         self.masked_rows_only = masked_rows_only           # graph decode: logits for still-masked positions only
         self._graphs = {}
@@ -540,6 +543,12 @@ class BlockDiffusionEngine:
             g["graph"].replay()
         return g["hidden"], g
 
+    def _noise(self, logits):
+        if self.gumbel is None:
+            return None
+        e = torch.empty(logits.shape, dtype=torch.float32, device=logits.device).exponential_(generator=self.gumbel)
+        return -e.log_()
+
     def _temperatures(self, seqs):
         key = tuple(s.temperature for s in seqs)
         if self._temps is None or self._temps[0] != key:
@@ -557,8 +566,9 @@ class BlockDiffusionEngine:
             x = g["ids"][:len(seqs)]
         else:
             x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
+        extra = {} if self.gumbel is None else {"noise": self._noise(logits)}
         _, _, transfer, _n = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
-                                         temperatures=self._temperatures(seqs))
+                                         temperatures=self._temperatures(seqs), **extra)
         if g is None:
             x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
             for i, s in enumerate(seqs):
@@ -630,7 +640,7 @@ class BlockDiffusionEngine:
             temps = temps[:1]
         else:
             temps = temps.index_select(0, idx_dev // S)
-        x0_rows, p_rows = confidence_argmax(logits, temps)
+        x0_rows, p_rows = confidence_argmax(logits, temps, self._noise(logits))
         if "x0" not in g:
             g["x0"] = torch.zeros(g["ids"].numel(), dtype=torch.int64, device=self.device)
             g["x0_p"] = torch.zeros(g["ids"].numel(), dtype=torch.float32, device=self.device)
