@@ -34,7 +34,6 @@ namespace {
 using namespace mdx_attn;
 
 constexpr int kMaxSq = 32;
-constexpr int kThreads = 256;      // 4 wavefronts, 2 workgroups per CU
 constexpr int kChunkAlign = 256;   // split boundaries are multiples of this many keys
 
 __device__ __forceinline__ int wave_sum(int x) {
@@ -63,10 +62,15 @@ struct PagedParams {
     float* span_out;
 };
 
-template <int HPW, int DEPTH>
-__global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const PagedParams P)
+// WAVES = 4 (two workgroups per CU) or 8 (one workgroup per CU, 128-key tiles: for launches with about
+// one workgroup per CU, where a CU would otherwise hold four wavefronts only).
+template <int HPW, int DEPTH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_attn_kernel(const PagedParams P)
 {
-    constexpr int KW = 4 / HPW;                     // key slices (wavefronts per head)
+    constexpr int kThreads = 64 * WAVES;
+    constexpr int kRowsPerPass = kThreads / 16;     // LDS rows one pass of the workgroup stages
+    constexpr int kPassesPerSlice = 32 / kRowsPerPass;
+    constexpr int KW = WAVES / HPW;                 // key slices (wavefronts per head)
     constexpr int kTileKeys = 32 * KW;
     constexpr int kTileBytes = kTileKeys * kLdsPitch;
     constexpr int kPasses = TileRegs<kTileKeys, kThreads>::kPasses;   // 16 rows per pass
@@ -96,16 +100,24 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         }
         int n = 0;                                  // splits of sequence `lane` (padding rows get one)
         if (lane < P.bs) n = max(1, (ctx_l + span - 1) / span);
-        int before = 0;
-        for (int s = 0; s < P.bs; ++s) {
-            const int ns = __builtin_amdgcn_readlane(n, s);
-            before += s < lane ? ns : 0;
+        // Launch order: the first split of every sequence, then the second of those that have one, ...
+        // The last split of a sequence is its short remainder, so the workgroups that start late
+        // (when there are more of them than the chip holds at once) are the short ones.
+        int j = blockIdx.y, level = 0;
+        b = -1;
+        for (; level < P.nsplit; ++level) {
+            const unsigned long long has = __ballot(n > level);
+            const int c = __popcll(has);
+            if (j < c) {
+                const int before = __popcll(has & ((1ull << lane) - 1ull));
+                const unsigned long long hit = __ballot(((has >> lane) & 1ull) != 0 && before == j);
+                b = __ffsll((long long)hit) - 1;
+                break;
+            }
+            j -= c;
         }
-        const int j = blockIdx.y;
-        const unsigned long long le = __ballot(lane < P.bs && before <= j);
-        b = __popcll(le) - 1;
-        split = j - __builtin_amdgcn_readlane(before, b);
-        if (split >= __builtin_amdgcn_readlane(n, b)) return;   // past the last pair
+        if (b < 0) return;                          // past the last (sequence, split) pair
+        split = level;
     } else {
         b = blockIdx.y / P.nsplit;
         split = blockIdx.y % P.nsplit;
@@ -135,9 +147,9 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
     st.init();
 
     const int32_t* bt = P.block_table + (int64_t)b * P.bt_stride;
-    const int chunk = tid & 15, trow = tid >> 4;    // 256 threads: one pass stages 16 rows
+    const int chunk = tid & 15, trow = tid >> 4;    // one pass stages kRowsPerPass rows
     const int n_tiles = (key_end - key_begin + kTileKeys - 1) / kTileKeys;
-    // 16 consecutive keys starting at a multiple of 16 never straddle a page (page_size % 32 == 0):
+    // kRowsPerPass (16 or 32) consecutive keys starting at a multiple of that never straddle a page (page_size % 32 == 0):
     // each pass looks its page up once.  The loads are unconditional (rows past the context or on
     // an invalid page id read row `trow` of page 0 instead and are zeroed when they reach LDS), so
     // the number of loads in flight is known exactly and waiting for one register set does not
@@ -154,7 +166,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         sg.pass_ok = 0;
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
-            const int kp = key0 + 16 * p;
+            const int kp = key0 + kRowsPerPass * p;
             const int page_slot = P.page_shift >= 0 ? kp >> P.page_shift : kp / P.page_size;
             const int in_page = P.page_shift >= 0 ? kp & (P.page_size - 1) : kp % P.page_size;
             const bool inside = kp < key_end && page_slot < P.max_pages;
@@ -179,7 +191,7 @@ __global__ __launch_bounds__(kThreads, 2) void paged_block_attn_kernel(const Pag
         const char* lk = lds[t & 1];
         const int key0 = key_begin + t * kTileKeys + kw * 32;        // this wavefront's 32 keys = passes 2kw, 2kw+1
         // keys of an invalid page are excluded (not merely zeroed): the owning wavefront skips them
-        if ((tile_pass_ok[t & 1] >> (2 * kw)) & 1u) {
+        if ((tile_pass_ok[t & 1] >> (kPassesPerSlice * kw)) & 1u) {
             if (key0 + 32 <= key_end)
                 attn_step<1, 1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
             else
@@ -356,7 +368,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // kernel is fastest with 1.5 to 1.8 workgroups per CU in total (just under the two per CU that are
 // resident at once: one round, no tail of late workgroups), with splits of at least 512 keys (a
 // workgroup's fixed cost is worth some 300 keys of streaming) and with whole sequences once there
-// is a (sequence, head group) pair per CU (in the engine's decode pass at batch 32 that beats two
+// are about as many (sequence, head group) pairs as CUs (from 192 pairs on) (in the engine's decode pass at batch 32 that beats two
 // splits per sequence by 4 %: no partials to write, nothing to combine).  The host knows the
 // page-table width, not the lengths: tables are taken to be about 65 % full, and the last split of
 // a sequence to be half a split.  In the pair-per-CU case up to four splits per sequence are allowed
@@ -369,7 +381,7 @@ int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* devi
     const int64_t max_keys = (int64_t)max_pages * page_size;
     const int64_t whole = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;   // one split per sequence
     const double per_pair = 500.0 / ((double)bs * head_groups) - 0.5;                 // workgroups per pair
-    if ((int64_t)bs * head_groups >= 256 || per_pair <= 1.0) {
+    if ((int64_t)bs * head_groups >= 192 || per_pair <= 1.0) {
         if (bs > 64 || whole < 4 * kChunkAlign) return (int)whole;
         *device_span = true;
         return (int)((whole / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
@@ -464,8 +476,13 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     // the dense numbering never needs more than 2 bs (sequence, split) pairs, whatever nsplit allows.
     const int pairs_y = device_span ? (bs * P.nsplit < 2 * bs ? bs * P.nsplit : 2 * bs) : bs * P.nsplit;
     const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)pairs_y);
-    if (HPW == 2) paged_block_attn_kernel<2, 2><<<grid, kThreads, 0, stream>>>(P);
-    else          paged_block_attn_kernel<1, 1><<<grid, kThreads, 0, stream>>>(P);
+    // Up to one (sequence, head group) pair per CU: workgroups of 8 wavefronts on 128-key tiles, so that a
+    // CU that holds a single workgroup still has two wavefronts per SIMD (batch 32 x 8 KV heads: 79 -> 69 us
+    // on equal lengths); with more pairs than CUs the second round costs more than that gains.
+    const bool eight = device_span && (int64_t)bs * (num_q_heads / HPW) <= 256;
+    if (HPW == 2 && eight) paged_block_attn_kernel<2, 2, 8><<<grid, 512, 0, stream>>>(P);
+    else if (HPW == 2)     paged_block_attn_kernel<2, 2, 4><<<grid, 256, 0, stream>>>(P);
+    else                   paged_block_attn_kernel<1, 1, 4><<<grid, 256, 0, stream>>>(P);
     int rc = mdx::check_launch("paged_block_attn");
     if (rc != MDX_OK || P.nsplit == 1) return rc;
     paged_combine_kernel<<<(unsigned)(bs * num_q_heads), 256, 0, stream>>>(P);
