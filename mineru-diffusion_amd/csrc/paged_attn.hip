@@ -86,7 +86,8 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
     // ---- workgroup -> (sequence b, split) ------------------------------------------------------
     int b, split, span = P.chunk;
     if (P.bs <= 64) {
-        const int ctx_l = lane < P.bs ? max(0, P.context_lens[lane]) : 0;
+        // lengths beyond the page table name keys that do not exist: clipped here and below
+        const int ctx_l = lane < P.bs ? min(max(0, P.context_lens[lane]), P.max_pages * P.page_size) : 0;
         if (P.span_out) {
             // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
             // nothing to combine) -- unless one of them is much longer than the rest and would keep
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
         b = blockIdx.y / P.nsplit;
         split = blockIdx.y % P.nsplit;
     }
-    const int ctx = P.context_lens[b];
+    const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
     const int n_valid_splits = (ctx + span - 1) / span;
     if (ctx <= 0) {
         // graph-padding row: defined output (zeros), written by its split 0
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
 __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
     const int hq = blockIdx.x % P.num_q_heads, b = blockIdx.x / P.num_q_heads;
-    const int ctx = P.context_lens[b];
+    const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
     const int span = P.span_out ? (int)*P.span_out : P.chunk; // the attention kernel's choice
     const int nv = (ctx + span - 1) / span;
     if (nv <= 1) return;                                   // written directly by the attention kernel

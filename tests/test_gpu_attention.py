@@ -294,3 +294,22 @@ def test_paged_pair_per_cu_batches(dev):
     _check_paged(dev, ctxs, seed=61, pool=80)
     _check_paged(dev, [777] * 40, seed=62, pool=170)
     _check_paged(dev, [2048] * 32 + [0] * 8, seed=63, pool=270)
+
+
+def test_paged_length_beyond_the_page_table_is_clipped(dev):
+    """A context length larger than the page table can hold names keys that do not exist: the kernel
+    reads the table's pages only (and must not write partials outside its slots)."""
+    import mdx
+    g = torch.Generator().manual_seed(71)
+    q, kc, vc, bt, lens = _paged_inputs(g, [512, 700, 256], pool=12)
+    over = lens.clone()
+    over[0], over[2] = 5000, 300                       # table width is 3 pages = 768 keys
+    full = torch.tensor([bt.shape[1] * 256, 700, bt.shape[1] * 256], dtype=torch.int32)
+    bt2 = bt.clone()
+    bt2[0, 2] = bt[1, 2]                               # give the over-long rows a full table of valid pages
+    bt2[2, 1:] = bt[1, 1:]
+    scale = 1 / math.sqrt(128)
+    o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=over.to(dev), block_table=bt2.to(dev),
+                                    softmax_scale=scale, causal=False)
+    ref = oracle.paged_block_attn(q, kc, vc, bt2, torch.minimum(over, full), scale)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
