@@ -222,6 +222,22 @@ int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
                      int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream);
 
 /*
+ * The same with x given as `parts` partial products of the GEMM that made it (its K range cut
+ * into `parts` pieces, one batched GEMM): x_parts [parts, rows, hidden] in x_dtype MDX_BF16 or
+ * MDX_F32, part stride and row stride in elements; s = sum over parts (fp32, in order) +
+ * residual_in, then as above.  The reference calls one GEMM here (nanovllm/layers/linear.py:
+ * 150-153, 128-131); at a few hundred rows that GEMM has fewer tiles than the chip has CUs, and
+ * the sum of the partials costs nothing in a kernel that reads x anyway.  out may alias part 0
+ * only when x_dtype is MDX_BF16.
+ */
+int mdx_sum_add_rms_norm(const void* x_parts, int32_t parts, int64_t x_part_stride, int64_t x_row_stride, int32_t x_dtype,
+                         const void* residual_in, int64_t residual_in_row_stride,
+                         void* residual_out, int64_t residual_out_row_stride,
+                         const void* weight, float eps,
+                         void* out, int64_t out_row_stride,
+                         int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream);
+
+/*
  * SiluAndMul.forward of engines/nano_dvlm/nanovllm/layers/activation.py:7-16 (called at
  * nanovllm/models/sdar.py:110-111): x [rows, 2 * intermediate] -> out [rows, intermediate] =
  * round(silu(float(x[:, :I]))) * x[:, I:], the product rounded again.  Row strides in

@@ -104,27 +104,55 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     return q.view(*lead, num_q_heads, head_dim), None if k is None else k.view(*lead, num_kv_heads, head_dim), v
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None, *, parts: int = 0):
     """RMSNorm.forward (nanovllm/layers/layernorm.py:43-51): returns the normed x, or with a
-    residual the pair (normed x + residual, x + residual), in one launch."""
+    residual the pair (normed x + residual, x + residual), in one launch.
+
+    parts > 0: x is [parts, ..., hidden], the partial products of `linear_split_k` (bf16 or fp32),
+    summed in fp32 inside the same launch; weight, residual and the results are [..., hidden]."""
     _need_gpu(x, weight, residual)
     hidden = x.shape[-1]
-    assert x.stride(-1) == 1 and weight.shape == (hidden,) and weight.dtype == x.dtype and weight.is_contiguous()
-    x2 = x.reshape(-1, hidden)
-    out = torch.empty((x2.shape[0], hidden), dtype=x.dtype, device=x.device)
+    assert x.stride(-1) == 1 and weight.shape == (hidden,) and weight.is_contiguous()
+    shape = x.shape[1:] if parts else x.shape
+    if parts:
+        assert x.shape[0] == parts and x.dtype in (torch.bfloat16, torch.float32)
+        x3 = x.reshape(parts, -1, hidden)
+        x2, part_stride = x3[0], x3.stride(0)
+    else:
+        assert weight.dtype == x.dtype
+        x2, part_stride = x.reshape(-1, hidden), 0
+    out = torch.empty((x2.shape[0], hidden), dtype=weight.dtype, device=x.device)
     r2 = r_out = None
     if residual is not None:
-        assert residual.shape == x.shape and residual.dtype == x.dtype and residual.stride(-1) == 1
+        assert residual.shape == shape and residual.dtype == weight.dtype and residual.stride(-1) == 1
         r2 = residual.reshape(-1, hidden)
         r_out = torch.empty_like(out)
-    rc = _lib.lib().mdx_add_rms_norm(
-        x2.data_ptr(), x2.stride(0), r2.data_ptr() if r2 is not None else None, r2.stride(0) if r2 is not None else 0,
+    rc = _lib.lib().mdx_sum_add_rms_norm(
+        x2.data_ptr(), max(parts, 1), part_stride, x2.stride(0), _DTYPES[x.dtype],
+        r2.data_ptr() if r2 is not None else None, r2.stride(0) if r2 is not None else 0,
         r_out.data_ptr() if r_out is not None else None, r_out.stride(0) if r_out is not None else 0,
-        weight.data_ptr(), float(eps), out.data_ptr(), out.stride(0), x2.shape[0], hidden, _DTYPES[x.dtype], _stream(x))
+        weight.data_ptr(), float(eps), out.data_ptr(), out.stride(0), x2.shape[0], hidden, _DTYPES[weight.dtype], _stream(x))
     check(rc, "rms_norm")
     if residual is None:
-        return out.view(x.shape)
-    return out.view(x.shape), r_out.view(x.shape)
+        return out.view(shape)
+    return out.view(shape), r_out.view(shape)
+
+
+def linear_split_k(x: torch.Tensor, weight: torch.Tensor, parts: int, partial_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """x [..., K] times weight [N, K] transposed as `parts` partial products over equal slices of K,
+    made by ONE batched library GEMM over views of x and weight (nothing is copied): returns
+    [parts, ..., N], whose sum over dim 0 is F.linear(x, weight) (nanovllm/layers/linear.py:128-131,
+    150-153).  For GEMMs with few rows, whose output tiles would leave CUs idle; `rms_norm(...,
+    parts=parts)` adds the partials up.  partial_dtype torch.float32 keeps them unrounded."""
+    K, N = x.shape[-1], weight.shape[0]
+    assert weight.shape[1] == K and K % parts == 0 and x.is_contiguous() and weight.is_contiguous()
+    xa = x.reshape(-1, parts, K // parts).permute(1, 0, 2)            # [parts, M, K/parts], row stride K
+    wb = weight.view(N, parts, K // parts).permute(1, 2, 0)           # [parts, K/parts, N]
+    if partial_dtype is None or partial_dtype == x.dtype:
+        out = torch.bmm(xa, wb)
+    else:
+        out = torch.bmm(xa, wb, out_dtype=partial_dtype)
+    return out.view(parts, *x.shape[:-1], N)
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
