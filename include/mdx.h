@@ -126,6 +126,32 @@ int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void
                          void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
 
 /*
+ * The same in ONE launch where that pays: with about a (sequence, head group) pair per CU or
+ * more, where only sequences far longer than the rest are split, the last split of a pair to
+ * finish merges the pair's partials itself instead of a second (combine) launch; no workgroup
+ * waits for another.  In a decode pass whose sequences stay whole (the usual case at batch 32)
+ * this saves the launch of a kernel that finds nothing to do, 28 times per forward pass.  With
+ * fewer pairs, where every sequence is split, the call makes the same two launches as
+ * mdx_paged_block_attn (counting in costs each split workgroup a device-wide release).
+ *
+ * counters: mdx_paged_block_attn_counter_bytes(bs, Hq, Hkv) bytes of device memory, 4-byte
+ * aligned, that MUST BE ZERO before the first call and are left zero by every call that
+ * completes; calls that may run at the same time (different streams) need counters of their
+ * own.  workspace as above.  Same results bit for bit as mdx_paged_block_attn.
+ */
+int64_t mdx_paged_block_attn_counter_bytes(int32_t bs, int32_t num_q_heads, int32_t num_kv_heads);
+int mdx_paged_block_attn_single_launch(const void* q, void* o, const void* k_cache, const void* v_cache,
+                                       int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                                       int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                                       int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                                       const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                                       int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                                       int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                                       float scale, int32_t dtype,
+                                       void* workspace, int64_t workspace_bytes,
+                                       void* counters, int64_t counter_bytes, mdx_stream_t stream);
+
+/*
  * Confidence + argmax over the vocabulary -- replaces Sampler.prepare
  * (engines/nano_dvlm/nanovllm/layers/sampler.py:11-22).
  *

@@ -60,7 +60,65 @@ struct PagedParams {
     // through the scalar cache and wait on the vector-memory counter for them, draining the K/V
     // prefetch queue (measured: 78 -> 120 us).  Split sizes are far below 2^24, so the value is exact.
     float* span_out;
+    // Single-launch mode: one arrival counter per (sequence, head group), zero between launches.  The
+    // last split of a pair to arrive merges the pair's partials itself.  float for the same reason.
+    float* arrive;
 };
+
+// Merges the nv split partials of query s of (sequence b, head hq); the caller's 8 threads c = 0..7
+// of a query take 16 consecutive d values each.
+__device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, int nv)
+{
+    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
+    float M = kMinusBig, Lsum = 0.f;
+    float acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    for (int i0 = 0; i0 < nv; i0 += 4) {
+        float m[4], l[4];
+        float4 po[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t slot = slot0 + min(i0 + i, nv - 1);
+            m[i] = P.part_ml[(slot * 2 + 0) * kMaxSq + s];
+            l[i] = P.part_ml[(slot * 2 + 1) * kMaxSq + s];
+            const float4* src = reinterpret_cast<const float4*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) po[i][k] = src[k];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
+        const float Mn = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), M);
+        const float keep = __builtin_amdgcn_exp2f(M - Mn);
+        Lsum *= keep;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] *= keep;
+        M = Mn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool on = i0 + i < nv;
+            const float w = on ? __builtin_amdgcn_exp2f(m[i] - M) : 0.f;
+            Lsum += on ? w * l[i] : 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                acc[4 * k + 0] += on ? w * po[i][k].x : 0.f;
+                acc[4 * k + 1] += on ? w * po[i][k].y : 0.f;
+                acc[4 * k + 2] += on ? w * po[i][k].z : 0.f;
+                acc[4 * k + 3] += on ? w * po[i][k].w : 0.f;
+            }
+        }
+    }
+    const float inv = 1.0f / Lsum;
+    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+    __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        bf16x8_t out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (__bf16)(acc[8 * h + e] * inv);
+        *reinterpret_cast<bf16x8_t*>(dst + 8 * h) = out;
+    }
+}
 
 // WAVES = 4 (two workgroups per CU) or 8 (one workgroup per CU, 128-key tiles: for launches with about
 // one workgroup per CU, where a CU would otherwise hold four wavefronts only).
@@ -267,10 +325,11 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
         if (kw < stride) recv((wave / KW) * stride + kw);
         if (stride > 1) __syncthreads();
     }
-    if (kw != 0 || !row_ok) return;
+    const bool writer = kw == 0 && row_ok;
 
     // ---- output ---------------------------------------------------------------
     if (n_valid_splits == 1) {
+        if (!writer) return;
         const float inv = 1.0f / st.l[0];
         __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)r * P.o_ss + (int64_t)head * P.o_sh;
 #pragma unroll
@@ -283,7 +342,9 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
                 for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
                 *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
             }
-    } else {
+        return;
+    }
+    if (writer) {
         const int64_t slot = ((int64_t)b * P.num_q_heads + head) * P.nsplit + split;
         float* po = P.part_o + (slot * kMaxSq + r) * kHeadDim;
 #pragma unroll
@@ -298,6 +359,25 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_at
             P.part_ml[(slot * 2 + 1) * kMaxSq + r] = st.l[0];
         }
     }
+    if (!P.arrive) return;                       // two-launch mode: the combine kernel follows
+
+    // ---- single-launch mode: the last split of this (sequence, head group) to arrive merges them ----
+    // Release: every writer makes its partials visible device-wide before the workgroup counts
+    // itself in; acquire: the workgroup that finds itself last drops stale cache lines before it
+    // reads the others' partials.  Nobody waits for anybody: a workgroup that is not last leaves.
+    __shared__ int i_am_last;
+    __threadfence();
+    __syncthreads();
+    float* counter = P.arrive + (int64_t)b * gridDim.x + hg;
+    if (tid == 0) i_am_last = atomicAdd(counter, 1.0f) == (float)(n_valid_splits - 1) ? 1 : 0;
+    __syncthreads();
+    if (!i_am_last) return;
+    __threadfence();
+    for (int e = tid; e < HPW * 256; e += kThreads) {
+        const int s = (e & 255) >> 3;
+        if (s < P.sq) combine_query(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
+    }
+    if (tid == 0) *counter = 0.f;                // ready for the next launch
 }
 
 // One workgroup per (sequence, head): merges the split partials of its 32 queries; thread t takes
@@ -314,55 +394,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     if (nv <= 1) return;                                   // written directly by the attention kernel
     const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
     if (s >= P.sq) return;
-    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
-    float M = kMinusBig, Lsum = 0.f;
-    float acc[16];
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-    for (int i0 = 0; i0 < nv; i0 += 4) {
-        float m[4], l[4];
-        float4 po[4][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t slot = slot0 + min(i0 + i, nv - 1);
-            m[i] = P.part_ml[(slot * 2 + 0) * kMaxSq + s];
-            l[i] = P.part_ml[(slot * 2 + 1) * kMaxSq + s];
-            const float4* src = reinterpret_cast<const float4*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) po[i][k] = src[k];
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
-        const float Mn = fmaxf(fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3])), M);
-        const float keep = __builtin_amdgcn_exp2f(M - Mn);
-        Lsum *= keep;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[e] *= keep;
-        M = Mn;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const bool on = i0 + i < nv;
-            const float w = on ? __builtin_amdgcn_exp2f(m[i] - M) : 0.f;
-            Lsum += on ? w * l[i] : 0.f;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                acc[4 * k + 0] += on ? w * po[i][k].x : 0.f;
-                acc[4 * k + 1] += on ? w * po[i][k].y : 0.f;
-                acc[4 * k + 2] += on ? w * po[i][k].z : 0.f;
-                acc[4 * k + 3] += on ? w * po[i][k].w : 0.f;
-            }
-        }
-    }
-    const float inv = 1.0f / Lsum;
-    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-    __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        bf16x8_t out;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] = (__bf16)(acc[8 * h + e] * inv);
-        *reinterpret_cast<bf16x8_t*>(dst + 8 * h) = out;
-    }
+    combine_query(P, b, hq, s, c, nv);
 }
 
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
@@ -414,15 +446,18 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
     return (int64_t)bs * num_q_heads * nsplit * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;   // + the split size
 }
 
-extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void* v_cache,
-                                    int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
-                                    int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
-                                    int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
-                                    const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
-                                    int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
-                                    int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
-                                    float scale, int32_t dtype,
-                                    void* workspace, int64_t workspace_bytes, mdx_stream_t stream_)
+namespace {
+
+int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cache,
+                 int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                 int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                 int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                 const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                 int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                 int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                 float scale, int32_t dtype,
+                 void* workspace, int64_t workspace_bytes, bool single_launch, void* counters, int64_t counter_bytes,
+                 mdx_stream_t stream_)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && sq >= 0 && max_pages >= 0 && num_pages >= 0, MDX_EINVAL, "paged_block_attn: negative size");
@@ -460,7 +495,7 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     P.nsplit = nsplit_of(max_pages, page_size, P.chunk);
     P.num_q_heads = num_q_heads;
     P.c = scale * kLog2e;
-    P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr;
+    P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr; P.arrive = nullptr;
     if (P.nsplit > 1) {
         const int64_t n_slots = (int64_t)bs * num_q_heads * P.nsplit;
         const int64_t need = n_slots * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;
@@ -470,6 +505,18 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
         P.part_o = static_cast<float*>(workspace);
         P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
         if (device_span) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
+        // Counting in costs every split workgroup a device-wide release (a walk of its XCD's L2 for dirty
+        // lines), which a launch of hundreds of split workgroups pays a hundred times over (config 2:
+        // 48 -> 145 us), while a launch whose sequences stay whole pays nothing and saves the combine
+        // launch (batch 32: 62 -> 60 us).  So only the launches that cut nothing but outliers
+        // (device_span) take the single-launch path; the others keep the combine kernel.
+        if (single_launch && device_span) {
+            const int64_t need_c = (int64_t)bs * (num_q_heads / HPW) * (int64_t)sizeof(float);
+            MDX_REQUIRE(counters && counter_bytes >= need_c, MDX_EWORKSPACE,
+                        "paged_block_attn: %lld bytes of arrival counters needed, %lld given", (long long)need_c, (long long)counter_bytes);
+            MDX_REQUIRE(((uintptr_t)counters & 3) == 0, MDX_EWORKSPACE, "paged_block_attn: counters not 4-byte aligned");
+            P.arrive = static_cast<float*>(counters);
+        }
     }
     // head group fastest, then the dense (sequence, split) index
     MDX_REQUIRE((int64_t)bs * P.nsplit <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: bs * splits %lld > 65535", (long long)bs * P.nsplit);
@@ -485,7 +532,49 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
     else if (HPW == 2)     paged_block_attn_kernel<2, 2, 4><<<grid, 256, 0, stream>>>(P);
     else                   paged_block_attn_kernel<1, 1, 4><<<grid, 256, 0, stream>>>(P);
     int rc = mdx::check_launch("paged_block_attn");
-    if (rc != MDX_OK || P.nsplit == 1) return rc;
+    if (rc != MDX_OK || P.nsplit == 1 || P.arrive) return rc;
     paged_combine_kernel<<<(unsigned)(bs * num_q_heads), 256, 0, stream>>>(P);
     return mdx::check_launch("paged_combine");
+}
+
+}  // namespace
+
+extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void* v_cache,
+                                    int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                                    int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                                    int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                                    const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                                    int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                                    int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                                    float scale, int32_t dtype,
+                                    void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    return launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
+                        cache_stride_page, cache_stride_tok, cache_stride_head, block_table, bt_stride, context_lens,
+                        bs, sq, num_q_heads, num_kv_heads, head_dim, max_pages, page_size, num_pages, scale, dtype,
+                        workspace, workspace_bytes, false, nullptr, 0, stream);
+}
+
+extern "C" int64_t mdx_paged_block_attn_counter_bytes(int32_t bs, int32_t num_q_heads, int32_t num_kv_heads)
+{
+    if (bs <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return 0;
+    const int G = num_q_heads / num_kv_heads;
+    return (int64_t)bs * (num_q_heads / ((G % 2 == 0) ? 2 : 1)) * (int64_t)sizeof(float);
+}
+
+extern "C" int mdx_paged_block_attn_single_launch(const void* q, void* o, const void* k_cache, const void* v_cache,
+                                                  int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                                                  int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                                                  int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                                                  const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                                                  int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                                                  int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                                                  float scale, int32_t dtype,
+                                                  void* workspace, int64_t workspace_bytes,
+                                                  void* counters, int64_t counter_bytes, mdx_stream_t stream)
+{
+    return launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
+                        cache_stride_page, cache_stride_tok, cache_stride_head, block_table, bt_stride, context_lens,
+                        bs, sq, num_q_heads, num_kv_heads, head_dim, max_pages, page_size, num_pages, scale, dtype,
+                        workspace, workspace_bytes, true, counters, counter_bytes, stream);
 }

@@ -204,12 +204,37 @@ sparse_attn_varlen_v2 = sparse_attn_varlen
 
 
 # --------------------------------------------------------------------------- paged decode
+_arrival_counters: dict = {}          # device index -> zeroed fp32 counters of the single-launch mode
+
+
+def _paged_counters(device: torch.device, n_bytes: int):
+    """The per-device arrival counters of mdx_paged_block_attn_single_launch: zero when created, left
+    zero by every launch.  Launches on one device share them, which is safe as long as they do not
+    run at the same time (one stream at a time, as the engine works); callers that overlap paged
+    attention launches on several streams pass their own `counters=`.  None while a graph is being
+    captured and no buffer exists yet (it could not be zeroed outside the graph): the caller then
+    takes the two-launch entry point."""
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    buf = _arrival_counters.get(key)
+    if buf is None or buf.numel() * 4 < n_bytes:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        buf = torch.zeros(max(4096, n_bytes // 4), dtype=torch.float32, device=device)
+        _arrival_counters[key] = buf
+    return buf
+
+
 def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
                             cache_seqlens: torch.Tensor, block_table: torch.Tensor,
-                            softmax_scale: float | None = None, causal: bool = False) -> torch.Tensor:
+                            softmax_scale: float | None = None, causal: bool = False,
+                            counters: torch.Tensor | None | bool = None) -> torch.Tensor:
     """The subset of flash_attn.flash_attn_with_kvcache used at sdar_attention.py:50-55:
     q [bs, Sq, Hq, d], caches [pages, page, Hkv, d], block_table [bs, max_pages] int32,
-    cache_seqlens [bs] int32, non-causal.  Returns o like q."""
+    cache_seqlens [bs] int32, non-causal.  Returns o like q.
+
+    counters (keyword, not in the reference): None = single launch with this module's per-device
+    arrival counters; a zeroed fp32 tensor of the caller's = single launch with those (for launches
+    that may overlap on several streams); False = attention launch + combine launch."""
     if causal:
         raise MdxError("flash_attn_with_kvcache: only causal=False (block-diffusion decode) is implemented")
     _need_gpu(q, k_cache, v_cache, cache_seqlens, block_table)
@@ -227,13 +252,20 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     ws_bytes = L.mdx_paged_block_attn_workspace_bytes(bs, sq, hq, hkv, d, bt.shape[1], page)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     scale = 1.0 / math.sqrt(d) if softmax_scale is None else float(softmax_scale)
-    rc = L.mdx_paged_block_attn(
-        q.data_ptr(), o.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-        q.stride(0), q.stride(1), q.stride(2), o.stride(0), o.stride(1), o.stride(2),
-        k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
-        bt.data_ptr(), bt.stride(0), lens.data_ptr(),
-        bs, sq, hq, hkv, d, bt.shape[1], page, num_pages, scale, _DTYPES[q.dtype],
-        ws.data_ptr(), ws_bytes, _stream(q))
+    args = (q.data_ptr(), o.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+            q.stride(0), q.stride(1), q.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            k_cache.stride(0), k_cache.stride(1), k_cache.stride(2),
+            bt.data_ptr(), bt.stride(0), lens.data_ptr(),
+            bs, sq, hq, hkv, d, bt.shape[1], page, num_pages, scale, _DTYPES[q.dtype],
+            ws.data_ptr(), ws_bytes)
+    c_bytes = L.mdx_paged_block_attn_counter_bytes(bs, hq, hkv)
+    if counters is None:
+        counters = _paged_counters(q.device, c_bytes)
+    if counters is None or counters is False:
+        rc = L.mdx_paged_block_attn(*args, _stream(q))
+    else:
+        assert counters.dtype == torch.float32 and counters.is_contiguous() and counters.device == q.device
+        rc = L.mdx_paged_block_attn_single_launch(*args, counters.data_ptr(), counters.numel() * 4, _stream(q))
     check(rc, "flash_attn_with_kvcache")
     return o
 

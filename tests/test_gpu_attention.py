@@ -121,12 +121,22 @@ def _check_paged(dev, ctxs, seed=0, **kw):
     g = torch.Generator().manual_seed(seed)
     q, kc, vc, bt, lens = _paged_inputs(g, ctxs, **kw)
     scale = 1 / math.sqrt(q.shape[-1])
-    o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens.to(dev),
-                                    block_table=bt.to(dev), softmax_scale=scale, causal=False)
+    args = (q.to(dev), kc.to(dev), vc.to(dev))
+    kwargs = dict(cache_seqlens=lens.to(dev), block_table=bt.to(dev), softmax_scale=scale, causal=False)
+    o = mdx.flash_attn_with_kvcache(*args, **kwargs)                  # single launch, the module's counters
     torch.cuda.synchronize()
     ref = oracle.paged_block_attn(q, kc, vc, bt, lens, scale)
     err = (o.float().cpu() - ref).abs().max().item()
     assert err < TOL, f"max-abs {err} for ctxs={ctxs}"
+    # the attention + combine launches and the single launch (twice on the same counters, which every
+    # launch must leave zero) give the same bits
+    two = mdx.flash_attn_with_kvcache(*args, **kwargs, counters=False)
+    own = torch.zeros(4096, dtype=torch.float32, device=dev)
+    for _ in range(2):
+        one = mdx.flash_attn_with_kvcache(*args, **kwargs, counters=own)
+        torch.cuda.synchronize()
+        assert torch.equal(one, two) and torch.equal(o, two)
+        assert own.abs().sum().item() == 0
     return o
 
 
