@@ -6,8 +6,9 @@
 // coalesced loads, several in flight per lane, an online (max, sum-of-exp)
 // pair per lane that is only rescaled when a 16-byte chunk raises the running
 // maximum, wavefront shuffles and one LDS hop for the row reduction.  The
-// argmax is found without per-element index bookkeeping: a lane remembers the
-// first chunk that set its maximum and re-reads that one chunk at the end.
+// argmax is found without per-element index bookkeeping: a lane notes the
+// position of a new maximum only when a 16-byte chunk raises its running maximum,
+// while that chunk is still in registers.
 //
 // Semantics follow engines/nano_dvlm/nanovllm/layers/sampler.py:11-61 and
 // mineru_diffusion/modeling_mineru_diffusion.py:518-532.
