@@ -110,7 +110,7 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * kernel picks it from the lengths); its size comes from
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
  * contents need no initialisation.
- * Supported: d == 128, Sq*(Hq/Hkv) <= 64, page_size % 32 == 0, MDX_BF16.
+ * Supported: d == 128, Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0, MDX_BF16.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
                                              int32_t num_kv_heads, int32_t head_dim,

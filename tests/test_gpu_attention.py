@@ -323,3 +323,16 @@ def test_paged_length_beyond_the_page_table_is_clipped(dev):
                                     softmax_scale=scale, causal=False)
     ref = oracle.paged_block_attn(q, kc, vc, bt2, torch.minimum(over, full), scale)
     assert (o.float().cpu() - ref).abs().max().item() < TOL
+
+
+def test_paged_single_launch_merges_across_xcds(dev):
+    """Three head groups instead of eight: consecutive workgroups go to consecutive XCDs, so the splits
+    of one (sequence, head group) pair run on different XCDs, each with an L2 of its own, and the one
+    that merges them reads partials written through another L2.  64 sequences (192 pairs: the kernel
+    cuts only the outliers), several rounds with different outliers."""
+    for seed in range(4):
+        g = torch.Generator().manual_seed(90 + seed)
+        ctxs = [int(x) for x in torch.randint(150, 330, (64,), generator=g)]
+        for i in torch.randperm(64, generator=g)[:5].tolist():
+            ctxs[i] = int(torch.randint(1200, 2049, (1,), generator=g))
+        _check_paged(dev, ctxs, seed=90 + seed, hq=6, hkv=3, pool=140)
