@@ -1,0 +1,84 @@
+"""GPU parity on randomly drawn (but fixed-seed) shapes: batch sizes, lengths, head layouts, block
+and page sizes that the parametrised tests do not name one by one.  Every case is checked against
+the fp32 oracle (max-abs 2e-2) and, for the paged kernel, the one-launch call against the
+two-launch call bit for bit."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+HEADS = [(16, 8), (8, 8), (4, 1), (6, 3), (3, 1), (2, 1), (12, 4)]
+
+
+def test_prefill_random_shapes(dev):
+    import mdx
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        hq, hkv = HEADS[rng.integers(len(HEADS))]
+        S = int(2 ** rng.integers(0, 8))
+        B = int(rng.integers(1, 7))
+        lens = [int(x) for x in rng.integers(0, 400, B)]
+        if case % 4 == 0:
+            lens[rng.integers(B)] = int(rng.integers(400, 1500))
+        if sum(lens) == 0:
+            lens[0] = 5
+        g = torch.Generator().manual_seed(1000 + case)
+        N = sum(lens)
+        q = torch.randn(N, hq, 128, generator=g).bfloat16()
+        k = torch.randn(N, hkv, 128, generator=g).bfloat16()
+        v = torch.randn(N, hkv, 128, generator=g).bfloat16()
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        print(f"prefill case {case}: heads {hq}/{hkv} S {S} lens {lens}", flush=True)
+        o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S)
+        torch.cuda.synchronize()
+        ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
+        err = (o.float().cpu() - ref).abs().max().item()
+        assert err < TOL, f"case {case}: max-abs {err} (heads {hq}/{hkv}, S {S}, lens {lens})"
+
+
+def test_paged_random_shapes(dev):
+    import mdx
+    rng = np.random.default_rng(4048)
+    for case in range(28):
+        hq, hkv = HEADS[rng.integers(len(HEADS))]
+        page = int(rng.choice([32, 64, 128, 256, 512, 96]))
+        sq = int(rng.choice([32, 32, 32, 1, 7, 16]))
+        bs = int(rng.choice([1, 2, 3, 5, 8, 13, 24, 32, 40, 64, 70]))
+        top = int(rng.choice([200, 700, 2500]))
+        ctxs = [int(x) for x in rng.integers(0, top, bs)]
+        if case % 3 == 0:
+            ctxs[rng.integers(bs)] = int(rng.integers(top, 4 * top))
+        if max(ctxs) == 0:
+            ctxs[0] = 3
+        extra = int(rng.integers(0, 3))                         # unused table columns (-1)
+        pages = [(c + page - 1) // page for c in ctxs]
+        pool = sum(pages) + 3
+        g = torch.Generator().manual_seed(2000 + case)
+        q = torch.randn(bs, sq, hq, 128, generator=g).bfloat16()
+        kc = torch.randn(pool, page, hkv, 128, generator=g).bfloat16()
+        vc = torch.randn(pool, page, hkv, 128, generator=g).bfloat16()
+        perm = torch.randperm(pool, generator=g)
+        bt = torch.full((bs, max(1, max(pages)) + extra), -1, dtype=torch.int32)
+        at = 0
+        for b, n in enumerate(pages):
+            bt[b, :n] = perm[at:at + n].to(torch.int32)
+            at += n
+        lens = torch.tensor(ctxs, dtype=torch.int32)
+        scale = 1 / math.sqrt(128)
+        print(f"paged case {case}: heads {hq}/{hkv} page {page} sq {sq} bs {bs} max ctx {max(ctxs)} width {bt.shape[1]}", flush=True)
+        args = (q.to(dev), kc.to(dev), vc.to(dev))
+        kw = dict(cache_seqlens=lens.to(dev), block_table=bt.to(dev), softmax_scale=scale, causal=False)
+        own = torch.zeros(4096, dtype=torch.float32, device=dev)
+        one = mdx.flash_attn_with_kvcache(*args, **kw, counters=own)
+        two = mdx.flash_attn_with_kvcache(*args, **kw, counters=False)
+        torch.cuda.synchronize()
+        ref = oracle.paged_block_attn(q, kc, vc, bt, lens, scale)
+        err = (two.float().cpu() - ref).abs().max().item()
+        assert err < TOL, f"case {case}: max-abs {err}"
+        assert torch.equal(one, two), f"case {case}: one launch differs from two"
+        assert own.abs().sum().item() == 0
