@@ -121,9 +121,10 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
 }
 
 // WAVES = 4 (two workgroups per CU) or 8 (one workgroup per CU, 128-key tiles: for launches with about
-// one workgroup per CU, where a CU would otherwise hold four wavefronts only).
+// one workgroup per CU, where a CU would otherwise hold four wavefronts only).  Tiles hold 32 keys per
+// key slice (WAVES / HPW slices); two 64-key tile buffers fit a CU twice, two 128-key ones once.
 template <int HPW, int DEPTH, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) void paged_block_attn_kernel(const PagedParams P)
+__global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_block_attn_kernel(const PagedParams P)
 {
     constexpr int kThreads = 64 * WAVES;
     constexpr int kRowsPerPass = kThreads / 16;     // LDS rows one pass of the workgroup stages
