@@ -45,20 +45,38 @@ def ev_pair():
     return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
 
-def time_kernel(fn, warmup, iters):
-    """Average duration (ms) of fn's GPU work.  fn(i) must only enqueue work (no allocation, no
-    host sync); the `iters` calls are bracketed by ONE pair of HIP events recorded on the launch
-    stream (torch's current stream, which is where libmdx enqueues), so the quotient is the
-    back-to-back launch duration with the host running ahead of the GPU.  A second number,
-    the minimum over individually bracketed launches, is returned for reference."""
+def time_kernel(fn, warmup, iters, graph=False, before_timed=None):
+    """Average duration (ms) of fn's GPU work.  fn(i) must only enqueue work on torch's current
+    stream (no allocation, no host sync); the `iters` calls are bracketed by ONE pair of HIP events
+    recorded on that stream.  With graph=True the `iters` calls are first recorded into a HIP graph
+    and the events bracket one replay of it: the figure is then the back-to-back duration of the
+    launches themselves, whatever the host's launch rate (under a profiler the host falls behind
+    the GPU on legs that take two short launches per call).  before_timed() runs (untimed) right
+    before the timed launches, for legs whose calls consume their input.  A second number, the
+    minimum over individually bracketed launches, is returned for reference."""
     for _ in range(warmup):
         fn(0)
     torch.cuda.synchronize()
     a, b = ev_pair()
-    a.record()
-    for i in range(iters):
-        fn(i)
-    b.record()
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(iters):
+                fn(i)
+        g.replay()
+        torch.cuda.synchronize()
+        if before_timed is not None:
+            before_timed()
+        a.record()
+        g.replay()
+        b.record()
+    else:
+        if before_timed is not None:
+            before_timed()
+        a.record()
+        for i in range(iters):
+            fn(i)
+        b.record()
     torch.cuda.synchronize()
     avg = a.elapsed_time(b) / iters
     pairs = []
@@ -409,7 +427,7 @@ def main():
             attn(g3["q"], g3["k"], g3["v"])
         torch.cuda.synchronize()
         ms_step = (time.perf_counter() - t0) * 1e3 / K
-        attn_ms, attn_min = time_kernel(attn_only, 2, K)
+        attn_ms, attn_min = time_kernel(attn_only, 2, K, graph=True)
         result_ops["staircase_attn"] = dict(
             ms=round(attn_ms, 4), ms_min=round(attn_min, 4), tflops=round(work3["flops"] / attn_ms / 1e9, 2),
             roofline=dict(bound="mfma", achieved=round(work3["flops"] / attn_ms / 1e9, 2), peak=PEAK_MFMA_TFLOPS,
@@ -418,7 +436,7 @@ def main():
             # the same launch on all-zero q/k/v (same strides): less bit toggling, higher clock
             zf = torch.zeros(g3["q"].shape[0], (HQ + 2 * HKV) * D, dtype=torch.bfloat16, device=dev)
             z = (torch.zeros_like(g3["q"]), torch.zeros_like(g3["k"]), zf[:, (HQ + HKV) * D:].view(-1, HKV, D))
-            z_ms, _ = time_kernel(lambda i: attn_only(i, z), 2, K)
+            z_ms, _ = time_kernel(lambda i: attn_only(i, z), 2, K, graph=True)
             calibration["staircase_attn_zero_inputs"] = dict(tflops=round(work3["flops"] / z_ms / 1e9, 1), ms=round(z_ms, 4))
             del zf
             del z
@@ -433,13 +451,12 @@ def main():
             sets.append((f2[:, HQ * D:(HQ + HKV) * D].reshape(N, HKV, D).contiguous(), f2[:, (HQ + HKV) * D:].view(N, HKV, D),
                          torch.zeros_like(g3["k_cache"]), torch.zeros_like(g3["v_cache"])))
         num_slots = g3["k_cache"].shape[0] * PAGE
-        stream = raw_stream()
 
         def store_only(i):
             k, v, kc, vc = sets[i % 3]
             L.mdx_store_kvcache(k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0), kc.data_ptr(), vc.data_ptr(),
-                                g3["slots"].data_ptr(), N, HKV * D, 2, num_slots, stream)
-        st_ms, st_min = time_kernel(store_only, W, K)
+                                g3["slots"].data_ptr(), N, HKV * D, 2, num_slots, raw_stream())
+        st_ms, st_min = time_kernel(store_only, W, K, graph=True)
         gbs = work3["store_bytes"] / st_ms / 1e6
         result_ops["store_kvcache"] = dict(
             ms=round(st_ms, 4), ms_min=round(st_min, 4),
@@ -469,7 +486,7 @@ def main():
                                         c2["lens"].data_ptr(), bs2, S, HQ, HKV, D, maxp, PAGE, kc2.shape[0],
                                         1 / math.sqrt(D), 0, ws2.data_ptr(), ws_bytes, raw_stream())
             assert rc == 0
-        pg_ms, pg_min = time_kernel(paged, W, K)
+        pg_ms, pg_min = time_kernel(paged, W, K, graph=True)
         gbs = c2["work"]["bytes"] / pg_ms / 1e6
         result_ops["paged_block_attn"] = dict(
             ms=round(pg_ms, 4), ms_min=round(pg_min, 4), tflops=round(c2["work"]["flops"] / pg_ms / 1e9, 2),
@@ -505,7 +522,11 @@ def main():
                                    x0_4.data_ptr(), p_4.data_ptr(), tr_4.data_ptr(), cnt_4.data_ptr(), 32, S, VOCAB,
                                    ws4.data_ptr(), ws_bytes4, raw_stream())
             assert rc == 0
-        um_ms, um_min = time_kernel(unmask, W, K)
+        fresh4 = dtoks.clone()
+
+        def remask():                                   # every timed call starts from the masked blocks
+            dtoks.copy_(fresh4)
+        um_ms, um_min = time_kernel(unmask, W, K, graph=True, before_timed=remask)
         gbs = c4["bytes"] / um_ms / 1e6
         result_ops["unmask_step"] = dict(
             ms=round(um_ms, 4), ms_min=round(um_min, 4),
