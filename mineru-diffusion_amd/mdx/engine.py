@@ -518,7 +518,7 @@ class BlockDiffusionEngine:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         g["graph"] = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g["graph"]):
+        with torch.cuda.graph(g["graph"], stream=side):    # the stream of the warm-up: its per-stream buffers exist
             g["hidden"] = self.model(self.model.embed(g["ids"]), g["pos"])
         torch.cuda.synchronize()
         return g

@@ -204,17 +204,18 @@ sparse_attn_varlen_v2 = sparse_attn_varlen
 
 
 # --------------------------------------------------------------------------- paged decode
-_arrival_counters: dict = {}          # device index -> zeroed fp32 counters of the single-launch mode
+_arrival_counters: dict = {}          # (device index, stream) -> zeroed fp32 counters of the single-launch mode
 
 
 def _paged_counters(device: torch.device, n_bytes: int):
-    """The per-device arrival counters of mdx_paged_block_attn_single_launch: zero when created, left
-    zero by every launch.  Launches on one device share them, which is safe as long as they do not
-    run at the same time (one stream at a time, as the engine works); callers that overlap paged
-    attention launches on several streams pass their own `counters=`.  None while a graph is being
-    captured and no buffer exists yet (it could not be zeroed outside the graph): the caller then
-    takes the two-launch entry point."""
-    key = device.index if device.index is not None else torch.cuda.current_device()
+    """The arrival counters of mdx_paged_block_attn_single_launch that this module keeps: one buffer
+    per device and stream, zero when created, left zero by every launch.  Launches on one stream run
+    one after the other, so they can share a buffer; a HIP graph keeps using the buffer of the stream
+    it was captured on wherever it is replayed.  None while a graph is being captured and that
+    stream has no buffer yet (it could not be zeroed outside the graph): the caller then takes the
+    two-launch entry point -- run the forward once on the capture stream before capturing."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(device).cuda_stream)
     buf = _arrival_counters.get(key)
     if buf is None or buf.numel() * 4 < n_bytes:
         if torch.cuda.is_current_stream_capturing():
@@ -232,9 +233,9 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
     q [bs, Sq, Hq, d], caches [pages, page, Hkv, d], block_table [bs, max_pages] int32,
     cache_seqlens [bs] int32, non-causal.  Returns o like q.
 
-    counters (keyword, not in the reference): None = single launch with this module's per-device
-    arrival counters; a zeroed fp32 tensor of the caller's = single launch with those (for launches
-    that may overlap on several streams); False = attention launch + combine launch."""
+    counters (keyword, not in the reference): None = single launch with this module's arrival
+    counters (one buffer per device and stream); a zeroed fp32 tensor of the caller's = single
+    launch with those; False = attention launch + combine launch."""
     if causal:
         raise MdxError("flash_attn_with_kvcache: only causal=False (block-diffusion decode) is implemented")
     _need_gpu(q, k_cache, v_cache, cache_seqlens, block_table)
