@@ -74,6 +74,22 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 0, one, one, 2, 32, null) == -1       # k < 1
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 1, one, one, 2, 2000, null) == -2      # block too long
     assert L.mdx_confidence_argmax(one, 10, 0, null, 1, null, 0, one, one, 4, 20, null, 0, null) == -2   # stride < vocab
+    # the single-launch paged call: with about a pair per CU (32 sequences x 8 head groups) it needs the counters
+    big = ctypes.c_void_p(1 << 20)
+    ws32 = L.mdx_paged_block_attn_workspace_bytes(32, 32, 16, 8, 128, 17, 256)
+    sl = lambda counters, nbytes: L.mdx_paged_block_attn_single_launch(                          # noqa: E731
+        one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,
+        32, 32, 16, 8, 128, 17, 256, 100, 0.1, 0, big, ws32, counters, nbytes, null)
+    assert ws32 > 0 and L.mdx_paged_block_attn_counter_bytes(32, 16, 8) == 32 * 8 * 4
+    assert sl(null, 0) == -3 and b"counters" in L.mdx_last_error()
+    assert sl(one, 32 * 8 * 4 - 4) == -3
+    assert sl(ctypes.c_void_p(18), 4096) == -3 and b"aligned" in L.mdx_last_error()
+    # partial products for the norm: parts and their dtype are checked before anything else
+    sn = lambda parts, xdt: L.mdx_sum_add_rms_norm(one, parts, 4096, 2048, xdt, null, 0, null, 0, one, 1e-6, big, 2048,   # noqa: E731
+                                                   8, 2048, 0, null)
+    assert sn(0, 0) == -1 and sn(17, 0) == -1 and b"parts" in L.mdx_last_error()
+    assert sn(2, 1) == -2 and b"x dtype" in L.mdx_last_error()
+    assert L.mdx_sum_add_rms_norm(one, 2, 4096, 2048, 2, null, 0, null, 0, one, 1e-6, one, 2048, 8, 2048, 0, null) == -1   # fp32 x in place
 
 
 def test_ops_fail_loudly_off_gpu():
