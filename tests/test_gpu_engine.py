@@ -230,3 +230,26 @@ def test_split_k_projections_generate_like_one_gemm(dev, partials):
     assert (hidden[0] - hidden[1]).abs().max().item() < (0.05 if partials == "bf16" else 0.02)
     same = sum(int(a == b) for a, b in zip(*outs))
     assert same >= 60, f"only {same}/64 tokens agree"
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_preemption_on_the_device_keeps_the_tokens(dev, graphs):
+    """scheduler.py:44-63 on the GPU: with too few pages for both sequences to grow, one is preempted, its
+    pages freed, and it is prefilled again later together with the tokens it had committed (the
+    prefill then runs over a partly unmasked current block).  Both sequences must finish, and with
+    the tokens of a run that had pages to spare (a near-tie may flip with the changed pass order)."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for pages in (12, 4):
+        eng = BlockDiffusionEngine(model, num_pages=pages, shuffle_pages_seed=2, decode_graphs=graphs, max_model_len=1024)
+        sp = SamplingParams(max_new_tokens=288, ignore_eos=True, transfer_count=8)
+        s1 = eng.add_request([5 + (i * 7) % 900 for i in range(300)], sp)      # grows from 2 to 3 pages
+        s2 = eng.add_request([11 + (i * 13) % 900 for i in range(40)], sp)     # grows from 1 to 2 pages: 5 > 4 in total
+        eng.generate()
+        assert s1.num_completion_tokens == 288 and s2.num_completion_tokens == 288
+        assert (eng.stats.get("preemptions", 0) >= 1) == (pages == 4)
+        assert len(eng.block_manager.free) == pages and not eng.running and not eng.waiting
+        outs.append(s1.completion_token_ids + s2.completion_token_ids)
+    same = sum(int(a == b) for a, b in zip(*outs))
+    assert same >= 0.9 * len(outs[0]), f"only {same}/{len(outs[0])} tokens agree"
