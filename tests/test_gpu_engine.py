@@ -253,3 +253,25 @@ def test_preemption_on_the_device_keeps_the_tokens(dev, graphs):
         outs.append(s1.completion_token_ids + s2.completion_token_ids)
     same = sum(int(a == b) for a, b in zip(*outs))
     assert same >= 0.9 * len(outs[0]), f"only {same}/{len(outs[0])} tokens agree"
+
+
+def test_sequences_that_finish_at_different_times(dev):
+    """Five requests of different lengths and budgets: as they finish one by one the decode batch shrinks
+    through the captured sizes 8, 4, 2, 1 (padding rows in between), page tables and lengths change
+    under the graphs, and every sequence must still produce what the eager engine produces."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for graphs in (False, True):
+        eng = BlockDiffusionEngine(model, num_pages=24, shuffle_pages_seed=4, decode_graphs=graphs, max_model_len=1024)
+        seqs = []
+        for i, (n_prompt, budget) in enumerate(((17, 32), (250, 160), (64, 96), (300, 64), (5, 128))):
+            sp = SamplingParams(max_new_tokens=budget, ignore_eos=True, transfer_count=8)
+            seqs.append(eng.add_request([3 + (j * (5 + i)) % 900 for j in range(n_prompt)], sp))
+        eng.generate()
+        assert [s.num_completion_tokens for s in seqs] == [32, 160, 96, 64, 128]
+        if graphs:
+            assert {1, 2, 4, 8} <= set(eng._graphs)
+        outs.append([t for s in seqs for t in s.completion_token_ids])
+    same = sum(int(a == b) for a, b in zip(*outs))
+    assert same >= 0.95 * len(outs[0]), f"only {same}/{len(outs[0])} tokens agree"
