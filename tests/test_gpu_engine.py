@@ -275,3 +275,27 @@ def test_sequences_that_finish_at_different_times(dev):
         outs.append([t for s in seqs for t in s.completion_token_ids])
     same = sum(int(a == b) for a, b in zip(*outs))
     assert same >= 0.95 * len(outs[0]), f"only {same}/{len(outs[0])} tokens agree"
+
+
+def test_stop_token_ends_the_sequence_at_its_block(dev):
+    """scheduler.py:71-78: a sequence whose finished block holds a stop token ends with that block
+    (unless ignore_eos), whatever its token budget."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    prompt = [7 + (j * 3) % 900 for j in range(100)]
+    eng = BlockDiffusionEngine(model, num_pages=8, decode_graphs=True, max_model_len=1024)
+    free = eng.add_request(prompt, SamplingParams(max_new_tokens=160, ignore_eos=True, transfer_count=8))
+    eng.generate()
+    tokens = free.completion_token_ids
+    # the stop token: the one whose first appearance comes latest (the tiny random model repeats itself a lot)
+    first = {}
+    for i, t in enumerate(tokens):
+        first.setdefault(t, i)
+    stop, at = max(first.items(), key=lambda kv: kv[1])
+    end = (at // 32 + 1) * 32
+    eng = BlockDiffusionEngine(model, num_pages=8, decode_graphs=True, max_model_len=1024)
+    sp = SamplingParams(max_new_tokens=160, ignore_eos=False, transfer_count=8, stop_token_ids=(stop,))
+    s = eng.add_request(prompt, sp)
+    eng.generate()
+    assert s.num_completion_tokens == end and s.completion_token_ids == tokens[:end]
+    assert len(eng.block_manager.free) == 8
