@@ -40,10 +40,22 @@ struct StaircaseParams {
     const __bf16* q; const __bf16* k; const __bf16* v; __bf16* o;
     int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;   // element strides: token, head
     const int32_t* cu_seqlens;
+    int total_tokens;
     int batch, n_row_groups, num_q_heads, num_kv_heads;
     int log2_s;
     float c;                                                   // scale * log2(e)
 };
+
+// Sequence b's first token and length.  Bounds that do not describe a range inside the packed
+// tensors (decreasing, negative, past total_tokens) are clipped to one, so that no row outside
+// q/k/v/o is ever touched; what such a call computes is unspecified.
+__device__ __forceinline__ void seq_bounds(const StaircaseParams& P, int b, int& seq0, int& L)
+{
+    const int lo = min(max(P.cu_seqlens[b], 0), P.total_tokens);
+    const int hi = min(max(P.cu_seqlens[b + 1], lo), P.total_tokens);
+    seq0 = lo;
+    L = hi - lo;
+}
 
 // Workgroup -> (sequence b, row group rg) for the j-th (sequence, row group) pair in launch order.
 // Row groups are handed out heaviest-first (the last row group of a sequence attends to the most
@@ -59,7 +71,8 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
     if (P.batch <= 64) {
         int g = 0;                                             // row groups of sequence `lane`
         if (lane < P.batch) {
-            const int len = P.cu_seqlens[lane + 1] - P.cu_seqlens[lane];
+            int first, len;
+            seq_bounds(P, lane, first, len);
             if (len > 0) g = ((((len + (1 << P.log2_s) - 1) >> P.log2_s) << P.log2_s) + kRowsPerWg - 1) / kRowsPerWg;
         }
         int level = -1, f_level = 0;
@@ -101,8 +114,8 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     int b, rg;
     if (!locate_row_group(P, blockIdx.x / P.num_q_heads, lane, b, rg)) return;
 
-    const int seq0 = P.cu_seqlens[b];
-    const int L = P.cu_seqlens[b + 1] - seq0;
+    int seq0, L;
+    seq_bounds(P, b, seq0, L);
     if (L <= 0) return;
     const int S = 1 << P.log2_s;
     const int Lp = ((L + S - 1) >> P.log2_s) << P.log2_s;     // padded length
@@ -238,8 +251,8 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     int b, rg;
     if (!locate_row_group(P, item / n_hslots, lane, b, rg)) return;
 
-    const int seq0 = P.cu_seqlens[b];
-    const int L = P.cu_seqlens[b + 1] - seq0;
+    int seq0, L;
+    seq_bounds(P, b, seq0, L);
     if (L <= 0) return;
     const int S = 1 << P.log2_s;
     const int Lp = ((L + S - 1) >> P.log2_s) << P.log2_s;
@@ -339,6 +352,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.q_st = q_stride_t; P.q_sh = q_stride_h; P.k_st = k_stride_t; P.k_sh = k_stride_h;
     P.v_st = v_stride_t; P.v_sh = v_stride_h; P.o_st = o_stride_t; P.o_sh = o_stride_h;
     P.cu_seqlens = cu_seqlens_k;
+    P.total_tokens = (int)total_tokens;
     P.batch = batch;
     const int64_t max_l = max_seqlen < total_tokens ? max_seqlen : total_tokens;
     P.n_row_groups = (int)((max_l + staircase_size - 1 + rows_per_wg - 1) / rows_per_wg);

@@ -336,3 +336,21 @@ def test_paged_single_launch_merges_across_xcds(dev):
         for i in torch.randperm(64, generator=g)[:5].tolist():
             ctxs[i] = int(torch.randint(1200, 2049, (1,), generator=g))
         _check_paged(dev, ctxs, seed=90 + seed, hq=6, hkv=3, pool=140)
+
+
+def test_prefill_sequence_bounds_are_clipped_to_the_tensors(dev):
+    """cu_seqlens that run past the packed tensors (or backwards) are clipped to them: the call touches no
+    row outside q/k/v/o, and a sequence whose bounds were only too long is computed as the clipped one."""
+    import mdx
+    g = torch.Generator().manual_seed(81)
+    q, k, v, cu = _packed(g, [200], 4, 2)
+    good = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    long = torch.tensor([0, 250], dtype=torch.int32)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), long.to(dev), long.to(dev), 32)
+    assert torch.equal(o, good)
+    back = torch.tensor([0, 120, 60, 200], dtype=torch.int32)           # the second sequence runs backwards: empty;
+                                                                         # the third overlaps rows 60.. of the first
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), back.to(dev), back.to(dev), 32)
+    torch.cuda.synchronize()
+    ref = oracle.staircase_attn_varlen(q[:120], k[:120], v[:120], torch.tensor([0, 120], dtype=torch.int32), 32)
+    assert (o[:60].float().cpu() - ref[:60]).abs().max().item() < TOL
