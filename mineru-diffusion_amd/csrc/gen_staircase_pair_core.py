@@ -29,7 +29,7 @@ Loop iteration t (S is double-buffered, cb = t & 1).  The MFMA / fragment stream
 reads of the first fragments of iteration t+1 are issued during the last items of iteration t.
   items 0..15:  32 MFMAs of QK(t+1) -> S[1-cb]   ||  rescale check(t), P(t) = exp2(S[cb]) in place
   wait until tile t+2 (loaded two iterations ago) has landed, barrier (publishes it; everyone has left tile t-1)
-  items 16..31: 32 MFMAs of PV(t) + 8 of ones . P^T (row sums)  ||  loads of tile t+4 -> slot of
+  items 16..31: 32 MFMAs of PV(t) + 16 small ones (row sums)    ||  loads of tile t+4 -> slot of
                 tile t-1, row max of S[1-cb], fragment addresses of iteration t+1, addresses of tile t+5
 
 Physical registers (all clobbered; the compiler keeps v0..v15 and a128..a191, a224..a255 for operands):
@@ -51,7 +51,7 @@ DMA_PER_TILE = 8                   # global_load_lds instructions per wavefront 
 KA = [f"v{24 + i}" for i in range(8)]            # K fragment address of k-step ks (current slot)
 VA = [[f"v{32 + 4 * q + dt}" for dt in range(4)] for q in range(2)]   # V^T address [lo / hi][d tile]
 VPAD, VLPM1, JPL, NEG_INF = "v40", "v41", "v42", "v43"
-ONES = "v[52:55]"                                # A fragment of bf16 ones: an MFMA with it sums the rows of P^T
+ONES = "v[52:53]"                                # four bf16 ones: A operand of the row-sum MFMA (see lacc)
 MX = ["v48", "v49"]
 MREL = "v50"
 GK = [f"v{56 + i}" for i in range(4)]            # global byte offsets of the rows the next loads fetch
@@ -77,6 +77,11 @@ def ptup(b, h, u, t):
     return f"v[{r}:{r + 3}]"
 
 
+def phalf(b, h, u, t, half):
+    r = sreg(b, h, u, 8 * t) + 2 * half
+    return f"v[{r}:{r + 1}]"
+
+
 def negm(h, i=None):
     r = 192 + 16 * h
     return f"v[{r}:{r + 15}]" if i is None else f"v{r + i}"
@@ -87,10 +92,19 @@ def otup(h, dt):
     return f"a[{r}:{r + 15}]"
 
 
+L_REGS = 4
+
+
 def lacc(h, i=None):
-    """Row sums l of head h: every register of the tuple holds the sum of its lane's query."""
+    """Row sums l of head h.  v_mfma_f32_4x4x4_16b_bf16 with A = ones adds, in every lane, the lane's own
+    four B values to each of its four accumulator registers (16 independent 4x4 blocks of four lanes:
+    D[i][j] = sum_k B[k][j], and lane 4 b + j holds column j of block b in A, B and D alike).  A lane's P^T
+    operands all belong to its one query, so this is the horizontal add that the row sum needs, on the
+    matrix pipe, at 8 cycles per four values: 16 of them per 64-key tile (128 cycles) where multiplying
+    the 32x32x16 operands by a block of ones took 8 x 32 cycles.  Each lane sums the keys of its own half
+    of every k-step; the two halves of a query (lanes l and l + 32) are added in the epilogue."""
     r = 192 + 16 * h
-    return f"a[{r}:{r + 15}]" if i is None else f"a{r + i}"
+    return f"a[{r}:{r + L_REGS - 1}]" if i is None else f"a{r + i}"
 
 
 def ring(i):
@@ -259,7 +273,7 @@ def check_rescale(uid, cb, masked):
                 r = sreg(cb, h, u, i)
                 out.append(f"v_sub_f32_e32 v{r}, v{r}, {T[0]}")
         out.append("s_nop 15")                      # the MFMAs of the previous tile's PV have long finished; margin only
-        for i in range(64 + 16):
+        for i in range(64 + L_REGS):
             a = f"a{64 * h + i}" if i < 64 else lacc(h, i - 64)
             t = T[2 + (i & 3)]
             out.append(f"v_accvgpr_read_b32 {t}, {a}")
@@ -295,7 +309,8 @@ def pv_items(cb):
                                            f"ds_read_b64_tr_b16 {frag[2]}, {VA[1][dt]}{sfx}"]
         mf = lambda frag, u=u, t=t, dt=dt: [
             f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)] + (
-            [f"v_mfma_f32_32x32x16_bf16 {lacc(h)}, {ONES}, {ptup(cb, h, u, t)}, {lacc(h)}" for h in range(2)] if dt == 1 else [])
+            [f"v_mfma_f32_4x4x4_16b_bf16 {lacc(h)}, {ONES}, {phalf(cb, h, u, t, half)}, {lacc(h)}"
+             for half in range(2) for h in range(2)] if dt == 1 else [])
         items.append((rd, mf))
     return items
 
@@ -357,9 +372,9 @@ def prologue():
         for first, last in dma_ops(slot):
             out += first + ["s_nop 0"] + last
     out += load_offset_ops()
-    for i in range(4):
+    for i in range(2):
         out.append(f"v_mov_b32_e32 v{52 + i}, 0x3f803f80")
-    for i in list(range(128)) + list(range(192, 224)):
+    for i in list(range(128)) + [192 + 16 * h + j for h in range(2) for j in range(L_REGS)]:
         out.append(f"v_accvgpr_write_b32 a{i}, 0")
     out += [f"s_waitcnt vmcnt({2 * DMA_PER_TILE})", "s_barrier"]      # tiles 0 and 1 have landed
     # QK(0) with C = 0, then m = row max of tile 0: -m tuples and S[0] -= m
@@ -455,7 +470,10 @@ def epilogue():
     out = [".Lend_%=:", "s_waitcnt lgkmcnt(0)", "s_nop 15", "s_nop 15"]
     out += [f"v_cmp_ne_u32_e32 vcc, 0, %[ok]", f"s_and_saveexec_b64 {S_SAVE}, vcc"]
     for h in range(2):
-        out += [f"v_accvgpr_read_b32 {T[7]}, {lacc(h, 0)}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
+        # l = this lane's partial sum + that of the lane holding the other keys of the same query
+        out += [f"v_accvgpr_read_b32 {T[7]}, {lacc(h, 0)}", "s_nop 1", f"v_mov_b32_e32 {T[6]}, {T[7]}", "s_nop 1",
+                f"v_permlane32_swap_b32_e32 {T[7]}, {T[6]}", "s_nop 1",
+                f"v_add_f32_e32 {T[7]}, {T[7]}, {T[6]}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
         for dt in range(4):
             for g in range(4):
                 for e in range(4):
