@@ -90,6 +90,22 @@ def time_kernel(fn, warmup, iters, graph=False, before_timed=None):
     return float(avg), float(min(x.elapsed_time(y) for x, y in pairs))
 
 
+def op_entry(ms_graph, ms_single, bound, work, unit_div, peak, unit, extra=None):
+    """One entry of "ops".  ms_graph: average duration of a launch inside one replay of a HIP graph of
+    K back-to-back launches (launch gaps of the host excluded: the kernel's own time, what rocprofv3's
+    kernel trace averages); ms_single: the fastest of ten individually bracketed eager launches (what a
+    caller that launches one at a time sees, launch latency included).  `roofline` uses ms_graph,
+    `roofline_single_launch` ms_single."""
+    def roof(ms):
+        a = work / ms / unit_div
+        return dict(bound=bound, achieved=round(a, 2), peak=peak, unit=unit, frac=round(a / peak, 4), traffic=None)
+    d = dict(ms_graph=round(ms_graph, 4), ms_single=round(ms_single, 4))
+    d.update(extra or {})
+    d["roofline"] = roof(ms_graph)
+    d["roofline_single_launch"] = roof(ms_single)
+    return d
+
+
 def raw_stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -428,10 +444,7 @@ def main():
         torch.cuda.synchronize()
         ms_step = (time.perf_counter() - t0) * 1e3 / K
         attn_ms, attn_min = time_kernel(attn_only, 2, K, graph=True)
-        result_ops["staircase_attn"] = dict(
-            ms=round(attn_ms, 4), ms_min=round(attn_min, 4), tflops=round(work3["flops"] / attn_ms / 1e9, 2),
-            roofline=dict(bound="mfma", achieved=round(work3["flops"] / attn_ms / 1e9, 2), peak=PEAK_MFMA_TFLOPS,
-                          unit="TFLOP/s", frac=round(work3["flops"] / attn_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), traffic=None))
+        result_ops["staircase_attn"] = op_entry(attn_ms, attn_min, "mfma", work3["flops"], 1e9, PEAK_MFMA_TFLOPS, "TFLOP/s")
         if calibration is not None:
             # the same launch on all-zero q/k/v (same strides): less bit toggling, higher clock
             zf = torch.zeros(g3["q"].shape[0], (HQ + 2 * HKV) * D, dtype=torch.bfloat16, device=dev)
@@ -457,11 +470,7 @@ def main():
             L.mdx_store_kvcache(k.data_ptr(), v.data_ptr(), k.stride(0), v.stride(0), kc.data_ptr(), vc.data_ptr(),
                                 g3["slots"].data_ptr(), N, HKV * D, 2, num_slots, raw_stream())
         st_ms, st_min = time_kernel(store_only, W, K, graph=True)
-        gbs = work3["store_bytes"] / st_ms / 1e6
-        result_ops["store_kvcache"] = dict(
-            ms=round(st_ms, 4), ms_min=round(st_min, 4),
-            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        result_ops["store_kvcache"] = op_entry(st_ms, st_min, "hbm", work3["store_bytes"], 1e6, PEAK_HBM_GBS, "GB/s")
         del sets
         torch.cuda.empty_cache()
     mdx.reset_context()
@@ -487,12 +496,10 @@ def main():
                                         1 / math.sqrt(D), 0, ws2.data_ptr(), ws_bytes, raw_stream())
             assert rc == 0
         pg_ms, pg_min = time_kernel(paged, W, K, graph=True)
-        gbs = c2["work"]["bytes"] / pg_ms / 1e6
-        result_ops["paged_block_attn"] = dict(
-            ms=round(pg_ms, 4), ms_min=round(pg_min, 4), tflops=round(c2["work"]["flops"] / pg_ms / 1e9, 2),
-            mfma_frac=round(c2["work"]["flops"] / pg_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), sum_ctx=c2["work"]["sum_ctx"],
-            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        result_ops["paged_block_attn"] = op_entry(
+            pg_ms, pg_min, "hbm", c2["work"]["bytes"], 1e6, PEAK_HBM_GBS, "GB/s",
+            dict(tflops=round(c2["work"]["flops"] / pg_ms / 1e9, 2),
+                 mfma_frac=round(c2["work"]["flops"] / pg_ms / 1e9 / PEAK_MFMA_TFLOPS, 4), sum_ctx=c2["work"]["sum_ctx"]))
         del c2
         torch.cuda.empty_cache()
 
@@ -527,11 +534,7 @@ def main():
         def remask():                                   # every timed call starts from the masked blocks
             dtoks.copy_(fresh4)
         um_ms, um_min = time_kernel(unmask, W, K, graph=True, before_timed=remask)
-        gbs = c4["bytes"] / um_ms / 1e6
-        result_ops["unmask_step"] = dict(
-            ms=round(um_ms, 4), ms_min=round(um_min, 4),
-            roofline=dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                          frac=round(gbs / PEAK_HBM_GBS, 4), traffic=None))
+        result_ops["unmask_step"] = op_entry(um_ms, um_min, "hbm", c4["bytes"], 1e6, PEAK_HBM_GBS, "GB/s")
         del c4
         torch.cuda.empty_cache()
 
@@ -558,13 +561,15 @@ def main():
         except Exception as e:  # the side numbers are informative only
             cpu["other_ops"] = {"error": str(e)}
 
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/)
+    # HBM bytes per launch: NOT measured by this run (counters need the profiler); copied from the
+    # summary of the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command under profiles/
     tfile = ROOT / "profiles" / "hbm_traffic_per_call.txt"
     if tfile.exists():
         measured = json.loads("".join(l for l in tfile.read_text().splitlines(True) if not l.startswith("#")))
         for name, op in result_ops.items():
             if name in measured:
                 op["roofline"]["traffic"] = measured[name]["bytes"]
+                op["roofline"]["traffic_source"] = "profiles/hbm_traffic_per_call.txt"
     value = work3["flops"] / ms_step / 1e9 if ms_step == ms_step else None
     line = {
         "metric": "staircase-attn TFLOP/s (%MFMA peak) + block-diffusion decode tokens/s, 1 GPU",

@@ -32,8 +32,8 @@ extern "C" {
 #define MDX_EWORKSPACE   -3        /* workspace missing or too small */
 #define MDX_ELAUNCH      -4        /* the HIP runtime refused the launch */
 
-#define MDX_BF16 0                 /* element types of q/k/v/o, the caches and the logits */
-#define MDX_F16  1
+#define MDX_BF16 0                 /* q/k/v/o, the caches, the layer ops, the logits */
+#define MDX_F16  1                 /* logits only */
 #define MDX_F32  2                 /* logits only */
 
 typedef void* mdx_stream_t;        /* hipStream_t */
@@ -76,9 +76,12 @@ int mdx_store_kvcache(const void* key, const void* value,
  * sequence (:52-53, :98-102): query i sees key j iff
  * j <= ((i+pad)/S+1)*S-1-pad, pad = ceil(L/S)*S-L.  Hq % Hkv == 0 and
  * kv head = q head / (Hq/Hkv) (:34).  softmax(q k^T * scale) v with fp32
- * accumulation.  max_seqlen is an upper bound on the longest sequence (it
- * sizes the grid; total_tokens is always a valid bound).  Supported: d == 128,
- * dtype MDX_BF16.
+ * accumulation.  max_seqlen MUST be >= the longest sequence in cu_seqlens: it
+ * sizes the grid, and rows of a longer sequence beyond it are never computed
+ * (their o rows keep what they held; the lengths are on the device, so the
+ * call cannot check this).  total_tokens is always a valid bound; the
+ * reference interface has no such argument.  Supported: d == 128, dtype
+ * MDX_BF16.
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                               int64_t q_stride_t, int64_t q_stride_h,
@@ -105,7 +108,8 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * padding, model_runner.py:123); context_lens [bs] int32.  Every query of
  * sequence b sees keys 0..context_lens[b]-1 (non-causal).  Rows with
  * context_lens[b] == 0 (graph padding, model_runner.py:205-208) produce
- * zeros.  Page ids outside [0, num_pages) are treated as holding no keys.
+ * zeros.  Page ids outside [0, num_pages) are treated as holding no keys; a
+ * sequence whose pages are all invalid therefore also produces zeros.
  * The workspace holds the split-KV partial results (and the split size when the
  * kernel picks it from the lengths); its size comes from
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
@@ -161,7 +165,9 @@ int mdx_paged_block_attn_single_launch(const void* q, void* o, const void* k_cac
  * noise: optional [rows, vocab] fp32 added to logits/T before the argmax
  * (the Gumbel term of sampler.py:15-18, made an explicit input so the kernel
  * holds no RNG), or NULL for the plain argmax.  Outputs: x0[r] = first index
- * of the maximum (int64), x0_p[r] = softmax(logits/T)[x0[r]] (fp32).
+ * of the maximum (int64), x0_p[r] = softmax(logits/T)[x0[r]] (fp32).  A row
+ * without any finite logit (all -inf) has no softmax: x0 = 0, x0_p = 0, so
+ * that no selection rule commits it.
  * Workspace from mdx_confidence_argmax_workspace_bytes (may be 0 bytes: then
  * workspace may be NULL).
  */
@@ -246,22 +252,6 @@ int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
                      const void* weight, float eps,
                      void* out, int64_t out_row_stride,
                      int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream);
-
-/*
- * The same with x given as `parts` partial products of the GEMM that made it (its K range cut
- * into `parts` pieces, one batched GEMM): x_parts [parts, rows, hidden] in x_dtype MDX_BF16 or
- * MDX_F32, part stride and row stride in elements; s = sum over parts (fp32, in order) +
- * residual_in, then as above.  The reference calls one GEMM here (nanovllm/layers/linear.py:
- * 150-153, 128-131); at a few hundred rows that GEMM has fewer tiles than the chip has CUs, and
- * the sum of the partials costs nothing in a kernel that reads x anyway.  out may alias part 0
- * only when x_dtype is MDX_BF16.
- */
-int mdx_sum_add_rms_norm(const void* x_parts, int32_t parts, int64_t x_part_stride, int64_t x_row_stride, int32_t x_dtype,
-                         const void* residual_in, int64_t residual_in_row_stride,
-                         void* residual_out, int64_t residual_out_row_stride,
-                         const void* weight, float eps,
-                         void* out, int64_t out_row_stride,
-                         int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream);
 
 /*
  * SiluAndMul.forward of engines/nano_dvlm/nanovllm/layers/activation.py:7-16 (called at

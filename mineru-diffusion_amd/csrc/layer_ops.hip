@@ -27,8 +27,7 @@ constexpr int kNormThreads = 256;
 constexpr int kNormMaxVecs = 4;                  // 16-byte vectors per thread: rows up to 8192 elements
 
 struct NormParams {
-    const void* x; int64_t x_stride;                       // [parts][rows][hidden]: bf16, or fp32 when x_f32
-    int parts; int64_t x_part_stride; int x_f32;
+    const __bf16* x; int64_t x_stride;                     // [rows][hidden]
     const __bf16* residual_in; int64_t res_in_stride;      // null: plain rms_forward
     __bf16* residual_out; int64_t res_out_stride;          // null when residual_in is null
     const __bf16* weight; float eps;
@@ -38,8 +37,7 @@ struct NormParams {
 
 // One workgroup per row; thread t holds vectors t, t + 256, ... of the row in registers, so the
 // row is read once.  In-place use (out == x, residual_out == residual_in) is safe: a thread
-// writes only the elements it has read.  x may come as several partial products of a GEMM whose
-// K range was cut (parts > 1): they are summed in fp32, in order, before anything is rounded.
+// writes only the elements it has read.
 template <int VECS>
 __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(const NormParams P)
 {
@@ -53,29 +51,9 @@ __global__ __launch_bounds__(kNormThreads) void add_rms_norm_kernel(const NormPa
     for (int i = 0; i < VECS; ++i) {
         const int v = tid + i * kNormThreads;
         if (v < n_vec) {
-            const int64_t at = row * P.x_stride + 8 * v;
-            if (P.x_f32) {
-                const float* xf = static_cast<const float*>(P.x) + at;
-                const float4 a0 = *reinterpret_cast<const float4*>(xf), a1 = *reinterpret_cast<const float4*>(xf + 4);
-                s[i][0] = a0.x; s[i][1] = a0.y; s[i][2] = a0.z; s[i][3] = a0.w;
-                s[i][4] = a1.x; s[i][5] = a1.y; s[i][6] = a1.z; s[i][7] = a1.w;
-                for (int p = 1; p < P.parts; ++p) {
-                    const float4 b0 = *reinterpret_cast<const float4*>(xf + p * P.x_part_stride);
-                    const float4 b1 = *reinterpret_cast<const float4*>(xf + p * P.x_part_stride + 4);
-                    s[i][0] += b0.x; s[i][1] += b0.y; s[i][2] += b0.z; s[i][3] += b0.w;
-                    s[i][4] += b1.x; s[i][5] += b1.y; s[i][6] += b1.z; s[i][7] += b1.w;
-                }
-            } else {
-                const __bf16* xb = static_cast<const __bf16*>(P.x) + at;
-                const bf16x8 a = *reinterpret_cast<const bf16x8*>(xb);
+            const bf16x8 a = *reinterpret_cast<const bf16x8*>(P.x + row * P.x_stride + 8 * v);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) s[i][e] = (float)a[e];
-                for (int p = 1; p < P.parts; ++p) {
-                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xb + p * P.x_part_stride);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) s[i][e] += (float)b[e];
-                }
-            }
+            for (int e = 0; e < 8; ++e) s[i][e] = (float)a[e];
             if (P.residual_in) {
                 const bf16x8 r = *reinterpret_cast<const bf16x8*>(P.residual_in + row * P.res_in_stride + 8 * v);
                 bf16x8 nr;
@@ -135,19 +113,17 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const __bf16* x, int6
 
 }  // namespace
 
-namespace {
-
-int launch_add_rms_norm(const char* what, const void* x, int32_t parts, int64_t x_part_stride, int64_t x_row_stride, int32_t x_dtype,
-                        const void* residual_in, int64_t residual_in_row_stride,
-                        void* residual_out, int64_t residual_out_row_stride,
-                        const void* weight, float eps, void* out, int64_t out_row_stride,
-                        int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream_)
+extern "C" int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
+                                const void* residual_in, int64_t residual_in_row_stride,
+                                void* residual_out, int64_t residual_out_row_stride,
+                                const void* weight, float eps,
+                                void* out, int64_t out_row_stride,
+                                int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream_)
 {
+    const char* what = "add_rms_norm";
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(rows >= 0 && hidden > 0, MDX_EINVAL, "%s: bad size (rows %lld, hidden %d)", what, (long long)rows, hidden);
     MDX_REQUIRE(dtype == MDX_BF16, MDX_EUNSUPPORTED, "%s: dtype %d (only bf16)", what, dtype);
-    MDX_REQUIRE(x_dtype == MDX_BF16 || x_dtype == MDX_F32, MDX_EUNSUPPORTED, "%s: x dtype %d (bf16 or fp32)", what, x_dtype);
-    MDX_REQUIRE(parts >= 1 && parts <= 16, MDX_EINVAL, "%s: %d parts (1 to 16)", what, parts);
     MDX_REQUIRE(hidden % 8 == 0 && hidden <= 8 * kNormThreads * kNormMaxVecs, MDX_EUNSUPPORTED,
                 "%s: hidden %d (multiples of 8 up to %d)", what, hidden, 8 * kNormThreads * kNormMaxVecs);
     MDX_REQUIRE(eps >= 0.f, MDX_EINVAL, "%s: negative eps", what);
@@ -157,17 +133,14 @@ int launch_add_rms_norm(const char* what, const void* x, int32_t parts, int64_t 
                 "%s: residual_in and residual_out go together", what);
     MDX_REQUIRE(rows <= 0x7fffffffLL, MDX_EUNSUPPORTED, "%s: %lld rows", what, (long long)rows);
     MDX_REQUIRE(mdx::aligned16(x) && mdx::aligned16(out) && mdx::aligned16(weight) && mdx::aligned16(residual_in) && mdx::aligned16(residual_out) &&
-                x_row_stride % 8 == 0 && out_row_stride % 8 == 0 && (parts == 1 || x_part_stride % 8 == 0) &&
+                x_row_stride % 8 == 0 && out_row_stride % 8 == 0 &&
                 (!residual_in || (residual_in_row_stride % 8 == 0 && residual_out_row_stride % 8 == 0)),
                 MDX_EUNSUPPORTED, "%s: rows must be 16-byte aligned", what);
     MDX_REQUIRE(x_row_stride >= hidden && out_row_stride >= hidden &&
                 (!residual_in || (residual_in_row_stride >= hidden && residual_out_row_stride >= hidden)),
                 MDX_EINVAL, "%s: row stride smaller than the row", what);
-    MDX_REQUIRE(parts == 1 || x_part_stride >= hidden, MDX_EINVAL, "%s: part stride smaller than a row", what);
-    MDX_REQUIRE(x_dtype != MDX_F32 || (out != x && residual_out != x), MDX_EINVAL, "%s: fp32 x may not be written in place", what);
     NormParams P;
-    P.x = x; P.x_stride = x_row_stride;
-    P.parts = parts; P.x_part_stride = parts > 1 ? x_part_stride : 0; P.x_f32 = x_dtype == MDX_F32;
+    P.x = (const __bf16*)x; P.x_stride = x_row_stride;
     P.residual_in = (const __bf16*)residual_in; P.res_in_stride = residual_in_row_stride;
     P.residual_out = (__bf16*)residual_out; P.res_out_stride = residual_out_row_stride;
     P.weight = (const __bf16*)weight; P.eps = eps;
@@ -179,30 +152,6 @@ int launch_add_rms_norm(const char* what, const void* x, int32_t parts, int64_t 
     else if (vecs == 2) add_rms_norm_kernel<2><<<grid, kNormThreads, 0, stream>>>(P);
     else add_rms_norm_kernel<4><<<grid, kNormThreads, 0, stream>>>(P);
     return mdx::check_launch(what);
-}
-
-}  // namespace
-
-extern "C" int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
-                                const void* residual_in, int64_t residual_in_row_stride,
-                                void* residual_out, int64_t residual_out_row_stride,
-                                const void* weight, float eps,
-                                void* out, int64_t out_row_stride,
-                                int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream)
-{
-    return launch_add_rms_norm("add_rms_norm", x, 1, 0, x_row_stride, dtype, residual_in, residual_in_row_stride,
-                               residual_out, residual_out_row_stride, weight, eps, out, out_row_stride, rows, hidden, dtype, stream);
-}
-
-extern "C" int mdx_sum_add_rms_norm(const void* x_parts, int32_t parts, int64_t x_part_stride, int64_t x_row_stride, int32_t x_dtype,
-                                    const void* residual_in, int64_t residual_in_row_stride,
-                                    void* residual_out, int64_t residual_out_row_stride,
-                                    const void* weight, float eps,
-                                    void* out, int64_t out_row_stride,
-                                    int64_t rows, int32_t hidden, int32_t dtype, mdx_stream_t stream)
-{
-    return launch_add_rms_norm("sum_add_rms_norm", x_parts, parts, x_part_stride, x_row_stride, x_dtype, residual_in, residual_in_row_stride,
-                               residual_out, residual_out_row_stride, weight, eps, out, out_row_stride, rows, hidden, dtype, stream);
 }
 
 extern "C" int mdx_silu_and_mul(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride,

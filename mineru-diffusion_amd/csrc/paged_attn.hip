@@ -27,7 +27,6 @@
 //    (m, l, O) that a second, small kernel combines.
 #include "mdx_common.h"
 #include "attn_tile.h"
-#include <cstdlib>
 
 namespace {
 
@@ -108,7 +107,7 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
             }
         }
     }
-    const float inv = 1.0f / Lsum;
+    const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;   // no valid key at all (every page id invalid): zeros, like a context of 0
     typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
     __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
 #pragma unroll
@@ -331,7 +330,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     // ---- output ---------------------------------------------------------------
     if (n_valid_splits == 1) {
         if (!writer) return;
-        const float inv = 1.0f / st.l[0];
+        const float inv = st.l[0] > 0.f ? 1.0f / st.l[0] : 0.f;   // no valid key at all: zeros
         __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)r * P.o_ss + (int64_t)head * P.o_sh;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
@@ -409,9 +408,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // and the kernel itself, which sees the lengths, cuts only sequences well above the mean
 // (*device_span; the dense workgroup numbering that this needs exists for up to 64 sequences).
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* device_span) {
-    static const int forced = [] { const char* e = getenv("MDX_PAGED_CHUNK"); return e ? atoi(e) : 0; }();
     *device_span = false;
-    if (forced >= kChunkAlign && forced % kChunkAlign == 0) return forced;
     const int64_t max_keys = (int64_t)max_pages * page_size;
     const int64_t whole = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;   // one split per sequence
     const double per_pair = 500.0 / ((double)bs * head_groups) - 0.5;                 // workgroups per pair
@@ -447,8 +444,9 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
     return (int64_t)bs * num_q_heads * nsplit * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;   // + the split size
 }
 
-namespace {
+namespace mdx {
 
+// The launch behind every paged entry point of the library.
 int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cache,
                  int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
                  int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
@@ -538,7 +536,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     return mdx::check_launch("paged_combine");
 }
 
-}  // namespace
+}  // namespace mdx
 
 extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void* v_cache,
                                     int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
@@ -550,7 +548,7 @@ extern "C" int mdx_paged_block_attn(const void* q, void* o, const void* k_cache,
                                     float scale, int32_t dtype,
                                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
 {
-    return launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
+    return mdx::launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
                         cache_stride_page, cache_stride_tok, cache_stride_head, block_table, bt_stride, context_lens,
                         bs, sq, num_q_heads, num_kv_heads, head_dim, max_pages, page_size, num_pages, scale, dtype,
                         workspace, workspace_bytes, false, nullptr, 0, stream);
@@ -574,7 +572,7 @@ extern "C" int mdx_paged_block_attn_single_launch(const void* q, void* o, const 
                                                   void* workspace, int64_t workspace_bytes,
                                                   void* counters, int64_t counter_bytes, mdx_stream_t stream)
 {
-    return launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
+    return mdx::launch_paged(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
                         cache_stride_page, cache_stride_tok, cache_stride_head, block_table, bt_stride, context_lens,
                         bs, sq, num_q_heads, num_kv_heads, head_dim, max_pages, page_size, num_pages, scale, dtype,
                         workspace, workspace_bytes, true, counters, counter_bytes, stream);

@@ -17,14 +17,8 @@
 
 namespace {
 
-#ifndef MDX_UNMASK_THREADS
-#define MDX_UNMASK_THREADS 256
-#endif
-#ifndef MDX_UNMASK_UNROLL
-#define MDX_UNMASK_UNROLL 2
-#endif
-constexpr int kThreads = MDX_UNMASK_THREADS;
-constexpr int kUnroll = MDX_UNMASK_UNROLL;   // 16-byte loads in flight per lane
+constexpr int kThreads = 256;
+constexpr int kUnroll = 2;               // 16-byte loads in flight per lane
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -3.0e38f;      // finite stand-in for -inf: keeps (m - m) away from inf - inf
 constexpr int kNoIndex = 0x7fffffff;
@@ -73,6 +67,20 @@ __device__ __forceinline__ Partial shfl_xor(const Partial& p, int mask, bool noi
         r.pick = kNegBig; r.pick_x = 0.f; r.pick_idx = kNoIndex;
     }
     return r;
+}
+
+// A row's final answer.  A row without any finite logit (all -inf) has no softmax: it reports
+// token 0 (where an argmax over equal values lands) with confidence 0, so no rule ever commits it.
+template <bool NOISE>
+__device__ __forceinline__ void finish_row(const Partial& r, float c, int64_t& x0, float& x0_p) {
+    if (r.idx == kNoIndex) { x0 = 0; x0_p = 0.f; return; }
+    if (NOISE) {
+        x0 = r.pick_idx;
+        x0_p = fast_exp2((r.pick_x - r.m) * c) / r.s;
+    } else {
+        x0 = r.idx;
+        x0_p = fminf(1.0f / r.s, 1.0f);          // the sum holds exp2(0) up to rounding
+    }
 }
 
 // --- element access by logits type: EPC = elements per 16-byte chunk ---------
@@ -261,12 +269,11 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
         for (int w = 1; w < kThreads / mdx::kWave; ++w) combine(r, wave_part[w], c, NOISE);
         if (nsplit > 1) {
             partials[row * nsplit + split] = r;
-        } else if (NOISE) {
-            x0[row] = r.pick_idx;
-            x0_p[row] = fast_exp2((r.pick_x - r.m) * c) / r.s;
         } else {
-            x0[row] = r.idx;
-            x0_p[row] = fminf(1.0f / r.s, 1.0f);      // the sum holds exp2(0) up to rounding
+            int64_t tok; float conf;
+            finish_row<NOISE>(r, c, tok, conf);
+            x0[row] = tok;
+            x0_p[row] = conf;
         }
     }
 }
@@ -284,13 +291,10 @@ __global__ __launch_bounds__(kThreads) void confidence_finalize_kernel(
     const float c = kLog2e / T_;
     Partial r = partials[row * nsplit];
     for (int s = 1; s < nsplit; ++s) combine(r, partials[row * nsplit + s], c, NOISE);
-    if (NOISE) {
-        x0[row] = r.pick_idx;
-        x0_p[row] = fast_exp2((r.pick_x - r.m) * c) / r.s;
-    } else {
-        x0[row] = r.idx;
-        x0_p[row] = fminf(1.0f / r.s, 1.0f);      // the sum holds exp2(0) up to rounding
-    }
+    int64_t tok; float conf;
+    finish_row<NOISE>(r, c, tok, conf);
+    x0[row] = tok;
+    x0_p[row] = conf;
 }
 
 // One workgroup per sequence; lane p owns block position p.  With FROM_PARTIALS the row splits
@@ -318,8 +322,7 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
             const float c = kLog2e / (temperatures ? temperatures[b] : 1.0f);
             Partial r = partials[at * nsplit];
             for (int s = 1; s < nsplit; ++s) combine(r, partials[at * nsplit + s], c, false);
-            pick = r.idx;
-            pick_p = fminf(1.0f / r.s, 1.0f);
+            finish_row<false>(r, c, pick, pick_p);
             x0[at] = pick;
             x0_p[at] = pick_p;
         } else {

@@ -11,8 +11,7 @@ reference functions they replace):
   Attention                 nanovllm/layers/sdar_attention.py:19-57
   Sampler                   nanovllm/layers/sampler.py:6-61
   Context / set_context ..  nanovllm/utils/context.py
-  rms_norm                  nanovllm/layers/layernorm.py:43-51 (RMSNorm.forward, with or without residual;
-                            optionally over the partial products of linear_split_k)
+  rms_norm                  nanovllm/layers/layernorm.py:43-51 (RMSNorm.forward, with or without residual)
   silu_and_mul              nanovllm/layers/activation.py:13-16 (SiluAndMul.forward)
   qk_norm_rope_store        nanovllm/models/sdar.py:79-83 in one launch (q/k norm, rotary, KV store)
 
@@ -22,7 +21,7 @@ without the built library or on a non-GPU tensor raises.
 from .context import Context, get_context, set_context, reset_context  # noqa: F401
 from .ops import (  # noqa: F401
     sparse_attn_varlen, sparse_attn_varlen_v2, store_kvcache, store_kvcache_maybe4d,
-    flash_attn_with_kvcache, confidence_argmax, select_transfer, unmask_step, qk_norm_rope_store, rms_norm, silu_and_mul, linear_split_k,
+    flash_attn_with_kvcache, confidence_argmax, select_transfer, unmask_step, qk_norm_rope_store, rms_norm, silu_and_mul,
 )
 from .layers import Attention, Sampler  # noqa: F401
 from ._lib import lib, library_path, MdxError  # noqa: F401

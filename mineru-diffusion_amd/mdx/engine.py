@@ -31,7 +31,7 @@ from torch import nn
 
 from .context import get_context, reset_context, set_context
 from .layers import Attention
-from .ops import (confidence_argmax, flash_attn_with_kvcache, linear_split_k, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
+from .ops import (confidence_argmax, flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
                   sparse_attn_varlen, unmask_step)
 
 PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
@@ -174,23 +174,6 @@ class DecoderConfig:
     mask_token_id: int = 151669
     fused_qk_rope_store: bool = True    # one libmdx launch for q/k norm + RoPE + KV store (else stock ops)
     fused_layer_ops: bool = True        # libmdx residual-add + RMSNorm and SiLU-and-multiply (else stock ops)
-    # Optional: passes of at most split_k_max_rows tokens (decode) run o_proj / down_proj as this many
-    # partial products over slices of K in one batched GEMM (their output alone has fewer tiles than the
-    # chip has CUs), and the residual-add + RMSNorm launch that follows sums the partials.  1 = one GEMM,
-    # as the reference computes it.  bf16 partials round each partial product once more than one GEMM
-    # does; "fp32" keeps them unrounded (and costs more traffic than the split saves at 1024 rows).
-    o_proj_split_k: int = 1
-    down_proj_split_k: int = 1
-    split_k_max_rows: int = 1024
-    split_k_partials: str = "bf16"
-
-
-class _Partials:
-    """[parts, ..., N] partial products of one projection, to be summed by the next norm launch."""
-    __slots__ = ("t",)
-
-    def __init__(self, t):
-        self.t = t
 
 
 def _rms(x, w, eps):
@@ -213,10 +196,8 @@ class DecoderLayer(nn.Module):
         self.attn = Attention(c.num_heads, c.head_dim, c.head_dim ** -0.5, c.num_kv_heads)
 
     def _norm(self, x, residual, w):
-        """layernorm.py:43-51: (normed, new residual).  x may be a _Partials of the GEMM before."""
+        """layernorm.py:43-51: (normed, new residual)."""
         c = self.c
-        if isinstance(x, _Partials):
-            return rms_norm(x.t, w, c.rms_norm_eps, residual, parts=x.t.shape[0])
         if c.fused_layer_ops:
             if residual is None:
                 return rms_norm(x, w, c.rms_norm_eps), x
@@ -239,7 +220,7 @@ class DecoderLayer(nn.Module):
             k = _rms(k, self.k_norm, c.rms_norm_eps)
             q, k = _rope(q, cos, sin), _rope(k, cos, sin)
             o = self.attn(q, k, v)
-        x = self._linear(o, self.o_proj, c.o_proj_split_k)
+        x = F.linear(o, self.o_proj)
         h, residual = self._norm(x, residual, self.post_attention_layernorm)
         gate_up = F.linear(h, self.gate_up_proj)
         if c.fused_layer_ops:
@@ -247,14 +228,7 @@ class DecoderLayer(nn.Module):
         else:
             gate, up = gate_up.chunk(2, dim=-1)
             act = F.silu(gate) * up
-        return self._linear(act, self.down_proj, c.down_proj_split_k), residual
-
-    def _linear(self, x, w, split):
-        """A projection whose output goes into a residual-add + RMSNorm launch."""
-        c = self.c
-        if split > 1 and c.fused_layer_ops and x.numel() // x.shape[-1] <= c.split_k_max_rows and x.is_contiguous():
-            return _Partials(linear_split_k(x, w, split, torch.float32 if c.split_k_partials == "fp32" else None))
-        return F.linear(x, w)
+        return F.linear(act, self.down_proj), residual
 
     def _attend_fused(self, qkv, positions, cos_table, sin_table):
         """sdar.py:79-83 + sdar_attention.py:34-57 with the q/k norm, RoPE and cache store done by
@@ -312,8 +286,6 @@ class Decoder(nn.Module):
         x, residual = inputs_embeds, None
         for layer in self.layers:
             x, residual = layer(positions, x, residual, cos, sin, self.cos, self.sin)
-        if isinstance(x, _Partials):
-            return rms_norm(x.t, self.norm, self.c.rms_norm_eps, residual, parts=x.t.shape[0])[0]
         if self.c.fused_layer_ops:
             return rms_norm(x, self.norm, self.c.rms_norm_eps, residual)[0]
         return _rms(x + residual, self.norm, self.c.rms_norm_eps)

@@ -104,31 +104,22 @@ def qk_norm_rope_store(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torc
     return q.view(*lead, num_q_heads, head_dim), None if k is None else k.view(*lead, num_kv_heads, head_dim), v
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None, *, parts: int = 0):
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.Tensor | None = None):
     """RMSNorm.forward (nanovllm/layers/layernorm.py:43-51): returns the normed x, or with a
-    residual the pair (normed x + residual, x + residual), in one launch.
-
-    parts > 0: x is [parts, ..., hidden], the partial products of `linear_split_k` (bf16 or fp32),
-    summed in fp32 inside the same launch; weight, residual and the results are [..., hidden]."""
+    residual the pair (normed x + residual, x + residual), in one launch."""
     _need_gpu(x, weight, residual)
     hidden = x.shape[-1]
-    assert x.stride(-1) == 1 and weight.shape == (hidden,) and weight.is_contiguous()
-    shape = x.shape[1:] if parts else x.shape
-    if parts:
-        assert x.shape[0] == parts and x.dtype in (torch.bfloat16, torch.float32)
-        x3 = x.reshape(parts, -1, hidden)
-        x2, part_stride = x3[0], x3.stride(0)
-    else:
-        assert weight.dtype == x.dtype
-        x2, part_stride = x.reshape(-1, hidden), 0
+    assert x.stride(-1) == 1 and weight.shape == (hidden,) and weight.is_contiguous() and weight.dtype == x.dtype
+    shape = x.shape
+    x2 = x.reshape(-1, hidden)
     out = torch.empty((x2.shape[0], hidden), dtype=weight.dtype, device=x.device)
     r2 = r_out = None
     if residual is not None:
         assert residual.shape == shape and residual.dtype == weight.dtype and residual.stride(-1) == 1
         r2 = residual.reshape(-1, hidden)
         r_out = torch.empty_like(out)
-    rc = _lib.lib().mdx_sum_add_rms_norm(
-        x2.data_ptr(), max(parts, 1), part_stride, x2.stride(0), _DTYPES[x.dtype],
+    rc = _lib.lib().mdx_add_rms_norm(
+        x2.data_ptr(), x2.stride(0),
         r2.data_ptr() if r2 is not None else None, r2.stride(0) if r2 is not None else 0,
         r_out.data_ptr() if r_out is not None else None, r_out.stride(0) if r_out is not None else 0,
         weight.data_ptr(), float(eps), out.data_ptr(), out.stride(0), x2.shape[0], hidden, _DTYPES[weight.dtype], _stream(x))
@@ -136,23 +127,6 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: torch.
     if residual is None:
         return out.view(shape)
     return out.view(shape), r_out.view(shape)
-
-
-def linear_split_k(x: torch.Tensor, weight: torch.Tensor, parts: int, partial_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """x [..., K] times weight [N, K] transposed as `parts` partial products over equal slices of K,
-    made by ONE batched library GEMM over views of x and weight (nothing is copied): returns
-    [parts, ..., N], whose sum over dim 0 is F.linear(x, weight) (nanovllm/layers/linear.py:128-131,
-    150-153).  For GEMMs with few rows, whose output tiles would leave CUs idle; `rms_norm(...,
-    parts=parts)` adds the partials up.  partial_dtype torch.float32 keeps them unrounded."""
-    K, N = x.shape[-1], weight.shape[0]
-    assert weight.shape[1] == K and K % parts == 0 and x.is_contiguous() and weight.is_contiguous()
-    xa = x.reshape(-1, parts, K // parts).permute(1, 0, 2)            # [parts, M, K/parts], row stride K
-    wb = weight.view(N, parts, K // parts).permute(1, 2, 0)           # [parts, K/parts, N]
-    if partial_dtype is None or partial_dtype == x.dtype:
-        out = torch.bmm(xa, wb)
-    else:
-        out = torch.bmm(xa, wb, out_dtype=partial_dtype)
-    return out.view(parts, *x.shape[:-1], N)
 
 
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
@@ -174,7 +148,10 @@ def sparse_attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seq
                        softmax_scale: float | None = None) -> torch.Tensor:
     """block_prefill_attention_v2.py:168-202: q [N, Hq, d], k/v [N, Hkv, d] packed over
     sequences, cu_seqlens int32 [B+1], blocks of `staircase_size` right-aligned; returns o like q.
-    max_seqlen (keyword, optional) only sizes the grid; the engine has it in its Context."""
+    max_seqlen (keyword, not in the reference) sizes the grid and must be >= the longest sequence:
+    rows beyond it are not computed, and the lengths live on the device, so this call cannot check
+    it.  None (the default) takes the total token count, which is always enough; the engine passes
+    the value it computed on the host while building cu_seqlens (Context.max_seqlen_k)."""
     _need_gpu(q, k, v, cu_seqlens_q, cu_seqlens_k)
     assert q.dim() == k.dim() == v.dim() == 3
     assert q.shape[0] == k.shape[0] == v.shape[0]
@@ -205,22 +182,27 @@ sparse_attn_varlen_v2 = sparse_attn_varlen
 
 # --------------------------------------------------------------------------- paged decode
 _arrival_counters: dict = {}          # (device index, stream) -> zeroed fp32 counters of the single-launch mode
+_COUNTER_FLOATS = 64 * 256            # the single-launch path exists for up to 64 sequences; 256 head groups is far beyond any model
 
 
 def _paged_counters(device: torch.device, n_bytes: int):
     """The arrival counters of mdx_paged_block_attn_single_launch that this module keeps: one buffer
     per device and stream, zero when created, left zero by every launch.  Launches on one stream run
     one after the other, so they can share a buffer; a HIP graph keeps using the buffer of the stream
-    it was captured on wherever it is replayed.  None while a graph is being captured and that
-    stream has no buffer yet (it could not be zeroed outside the graph): the caller then takes the
-    two-launch entry point -- run the forward once on the capture stream before capturing."""
+    it was captured on wherever it is replayed, which is why a buffer, once handed out, is never
+    replaced or freed: it has its full size from the start.  None when the request does not fit it,
+    or while a graph is being captured and that stream has no buffer yet (it could not be zeroed
+    outside the graph): the caller then takes the two-launch entry point -- run the forward once on
+    the capture stream before capturing."""
+    if n_bytes > _COUNTER_FLOATS * 4:
+        return None
     index = device.index if device.index is not None else torch.cuda.current_device()
     key = (index, torch.cuda.current_stream(device).cuda_stream)
     buf = _arrival_counters.get(key)
-    if buf is None or buf.numel() * 4 < n_bytes:
+    if buf is None:
         if torch.cuda.is_current_stream_capturing():
             return None
-        buf = torch.zeros(max(4096, n_bytes // 4), dtype=torch.float32, device=device)
+        buf = torch.zeros(_COUNTER_FLOATS, dtype=torch.float32, device=device)
         _arrival_counters[key] = buf
     return buf
 
@@ -259,9 +241,8 @@ def flash_attn_with_kvcache(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
             bt.data_ptr(), bt.stride(0), lens.data_ptr(),
             bs, sq, hq, hkv, d, bt.shape[1], page, num_pages, scale, _DTYPES[q.dtype],
             ws.data_ptr(), ws_bytes)
-    c_bytes = L.mdx_paged_block_attn_counter_bytes(bs, hq, hkv)
-    if counters is None:
-        counters = _paged_counters(q.device, c_bytes)
+    if counters is None:               # more than 64 sequences never take the single-launch path
+        counters = _paged_counters(q.device, L.mdx_paged_block_attn_counter_bytes(bs, hq, hkv)) if bs <= 64 else False
     if counters is None or counters is False:
         rc = L.mdx_paged_block_attn(*args, _stream(q))
     else:

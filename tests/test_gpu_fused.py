@@ -167,50 +167,3 @@ def test_silu_and_mul_matches_oracle(dev, rows, inter):
     # rows taken out of a wider matrix
     wide = (torch.randn(rows, 2 * inter + 64, generator=g)).bfloat16().to(dev)
     _ulp_close(mdx.silu_and_mul(wide[:, 64:]), oracle.silu_and_mul(wide[:, 64:].cpu()), frac_equal=0.97)
-
-
-@pytest.mark.parametrize("parts,pdtype", [(2, torch.bfloat16), (4, torch.bfloat16), (2, torch.float32), (4, torch.float32), (3, torch.bfloat16)])
-def test_rms_norm_sums_partial_products(dev, parts, pdtype):
-    """x given as partial products [parts, rows, hidden]: the launch sums them in fp32 (in order), then
-    adds the residual and norms as with one x.  Checked against the oracle on the fp32 sum: the new
-    residual bit for bit, the normed rows to one bf16 rounding."""
-    import mdx
-    g = torch.Generator().manual_seed(300 + parts)
-    rows, hidden = 70, 2048
-    xs = (torch.randn(parts, rows, hidden, generator=g)).to(pdtype)
-    res = torch.randn(rows, hidden, generator=g).bfloat16()
-    w = (1 + 0.1 * torch.randn(hidden, generator=g)).bfloat16()
-    total = xs[0].float()
-    for p in range(1, parts):
-        total = total + xs[p].float()                    # the kernel's order of additions
-    out, new_res = mdx.rms_norm(xs.to(dev), w.to(dev), 1e-6, res.to(dev), parts=parts)
-    s = total + res.float()
-    assert torch.equal(new_res.cpu(), s.bfloat16())
-    inv = torch.rsqrt((s.double() ** 2).mean(-1, keepdim=True) + 1e-6).float()
-    ref = ((s * inv).bfloat16().float() * w.float()).bfloat16()
-    diff = (out.cpu().float() - ref.float()).abs()
-    assert (diff <= 2.0 ** -7 * ref.float().abs() + 1e-30).all()
-    assert (out.cpu() == ref).float().mean().item() > 0.97
-    # without a residual (the plain norm of a sum)
-    out2 = mdx.rms_norm(xs.to(dev), w.to(dev), 1e-6, parts=parts)
-    inv2 = torch.rsqrt((total.double() ** 2).mean(-1, keepdim=True) + 1e-6).float()
-    ref2 = ((total * inv2).bfloat16().float() * w.float()).bfloat16()
-    assert ((out2.cpu().float() - ref2.float()).abs() <= 2.0 ** -7 * ref2.float().abs() + 1e-30).all()
-
-
-def test_linear_split_k_matches_linear(dev):
-    """The batched GEMM over K slices: the fp32 partials add up to the one-GEMM product within
-    accumulation-order noise, and nothing is copied (views of x and the weight)."""
-    import mdx
-    from mdx.ops import linear_split_k
-    g = torch.Generator().manual_seed(77)
-    x = torch.randn(4, 32, 6144, generator=g).bfloat16().to(dev)
-    w = (torch.randn(2048, 6144, generator=g) * 0.02).bfloat16().to(dev)
-    ref = torch.nn.functional.linear(x.float(), w.float())
-    for parts in (2, 4):
-        p32 = linear_split_k(x, w, parts, torch.float32)
-        assert p32.shape == (parts, 4, 32, 2048) and p32.dtype == torch.float32
-        assert (p32.sum(0) - ref).abs().max().item() < 2e-3
-        pb = linear_split_k(x, w, parts)
-        assert pb.dtype == torch.bfloat16
-        assert (pb.float().sum(0) - ref).abs().max().item() < 0.05
