@@ -44,6 +44,12 @@ def _engine_rule(conf: np.ndarray, masked: np.ndarray, threshold: float) -> np.n
 
 
 def _sampler_case(seed=21, bs=6):
+    logits, tokens, temps = _sampler_case6(seed)
+    return logits[:bs].contiguous(), tokens[:bs].contiguous(), temps[:bs].contiguous()
+
+
+def _sampler_case6(seed):
+    bs = 6
     g = torch.Generator().manual_seed(seed)
     logits = (torch.randn(bs, S, V, generator=g) * 3).bfloat16()
     logits[0, 3, 777] += 40.0                       # two positions far above the threshold in sequence 0
@@ -82,8 +88,9 @@ def test_sampler_forward_mutates_sequences_like_the_reference(dev, k):
 
 
 def test_sampler_forward_over_several_steps_unmasks_the_block(dev):
-    """The same Sequences through consecutive calls (as the scheduler re-schedules them): the block
-    empties in at most S steps with k = 1, the step map records the step of every commit."""
+    """The same Sequences through consecutive calls (as the scheduler re-schedules them): with k = 4 and
+    confidences below the threshold the block of 32 empties in exactly 8 steps, and the step map records
+    the step of every commit."""
     import mdx
     logits, tokens, temps = _sampler_case(seed=5, bs=2)
     tokens[:] = MASK_ID
