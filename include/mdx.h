@@ -156,6 +156,29 @@ int mdx_paged_block_attn_single_launch(const void* q, void* o, const void* k_cac
                                        void* counters, int64_t counter_bytes, mdx_stream_t stream);
 
 /*
+ * mdx_paged_block_attn for callers that CANNOT ALLOCATE (code under HIP graph capture without an
+ * allocator, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference, whose call sites allocate freely.  Same arguments, kernels and results (bit for
+ * bit) as mdx_paged_block_attn, without the workspace: the split-KV partials go into a 40 MiB
+ * device array that is part of the library image (each GPU the library runs on holds it until
+ * the process ends).  Shapes whose partials need more (the size mdx_paged_block_attn_workspace_bytes
+ * reports; 32 sequences x 16 heads with page tables of 17 pages need 32.5 MiB, 64 such sequences
+ * 65 MiB) are refused with MDX_EWORKSPACE.
+ * The call itself allocates and frees nothing; the first call on each device looks the array's
+ * address up (hipGetSymbolAddress), so make that call outside graph capture.  All calls on one
+ * GPU share the array: calls that may overlap (different streams) race on it; calls on one
+ * stream do not.
+ */
+int mdx_paged_block_attn_static(const void* q, void* o, const void* k_cache, const void* v_cache,
+                                int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                                int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                                int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                                const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                                int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                                int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                                float scale, int32_t dtype, mdx_stream_t stream);
+
+/*
  * Confidence + argmax over the vocabulary -- replaces Sampler.prepare
  * (engines/nano_dvlm/nanovllm/layers/sampler.py:11-22).
  *

@@ -32,6 +32,7 @@ SIGNATURES = {
     "mdx_paged_block_attn_counter_bytes": (c_int64, [_I32] * 3),
     "mdx_paged_block_attn_single_launch": (c_int32, [_P, _P, _P, _P] + [_I64] * 9 + [_P, _I64, _P] + [_I32] * 7 + [_I64, _F, _I32,
                                                                                                                     _P, _I64, _P, _I64, _P]),
+    "mdx_paged_block_attn_static": (c_int32, [_P, _P, _P, _P] + [_I64] * 9 + [_P, _I64, _P] + [_I32] * 7 + [_I64, _F, _I32, _P]),
     "mdx_confidence_argmax_workspace_bytes": (c_int64, [_I64, _I64]),
     "mdx_confidence_argmax": (c_int32, [_P, _I64, _I32, _P, _I32, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _P]),
     "mdx_select_transfer": (c_int32, [_P, _P, _P, _I64, _F, _I32, _P, _P, _I32, _I32, _P]),
