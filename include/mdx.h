@@ -285,6 +285,60 @@ int mdx_add_rms_norm(const void* x, int64_t x_row_stride,
 int mdx_silu_and_mul(const void* x, int64_t x_row_stride, void* out, int64_t out_row_stride,
                      int64_t rows, int32_t intermediate, int32_t dtype, mdx_stream_t stream);
 
+/*
+ * Denoising-block state kept on the device between decode passes (one entry per sequence of the
+ * batch, "lane"): tokens [bs, block_len] int64 (the current block, mask_token_id where still masked),
+ * lens [bs] (committed tokens), phase [bs] (MDX_PHASE_*), step [bs], step_map [bs, block_len].
+ * With these three calls a decode pass is a fixed list of launches: no upload of pass inputs, no
+ * blocking download of results; the host reads the 16-byte status of a lane when it wants to.
+ */
+#define MDX_PHASE_IDLE      0      /* padding lane or finished sequence: stores nothing, attends to nothing */
+#define MDX_PHASE_DENOISING 1      /* block holds masked positions (SequenceStatus.RUNNING) */
+#define MDX_PHASE_CACHING   2      /* block complete; the next pass stores its K/V (SequenceStatus.CACHING) */
+
+/*
+ * The pass inputs of ModelRunner.prepare_decode (engines/nano_dvlm/nanovllm/engine/model_runner.py:
+ * 169-185) computed on the device: positions[b, p] = lens[b] + p, slot_mapping[b, p] =
+ * block_table[b, t / page_size] * page_size + t % page_size with t = lens[b] + p (Sequence.get_slots,
+ * engine/sequence.py:117-141; -1 where the page table has no page), context_lens[b] = lens[b] +
+ * block_len.  Idle lanes get positions 0, slots -1, context 0 (the graph padding of
+ * model_runner.py:203-208).
+ */
+int mdx_block_prepare(const int32_t* lens, const int32_t* phase,
+                      const int32_t* block_table, int64_t bt_stride, int32_t max_pages,
+                      int32_t page_size, int32_t block_len,
+                      int64_t* positions, int32_t* slot_mapping, int32_t* context_lens,
+                      int32_t bs, mdx_stream_t stream);
+
+/*
+ * rows_out[i] = flat index b * block_len + p of the i-th still-masked position of the denoising lanes,
+ * in order; entries from the count up to rows_cap repeat entry 0 (0 when nothing is masked), so that
+ * a consumer of fixed size rows_cap may process them all; *n_rows_out = the count (entries beyond
+ * rows_cap are dropped: the caller sizes rows_cap from a bound it knows).  The sampler looks at the
+ * logits of masked positions only (layers/sampler.py:39,54).
+ */
+int mdx_masked_rows(const int64_t* tokens, const int32_t* phase, int64_t mask_token_id,
+                    int32_t bs, int32_t block_len,
+                    int64_t* rows_out, int32_t rows_cap, int32_t* n_rows_out, mdx_stream_t stream);
+
+/*
+ * After mdx_select_transfer: the rest of Sampler.forward (layers/sampler.py:56-59: step_map[transfer] =
+ * step, step += 1) and Scheduler.postprocess (engine/scheduler.py:65-82) per lane.  A denoising lane
+ * whose block has no masked position left becomes caching; a caching lane (this pass has stored its
+ * block's K/V) appends the block to out_tokens / out_steps [bs, out_stride] at offset lens - first_len
+ * (Sequence.append_block, engine/sequence.py:97-101), adds block_len to lens, refills the block with
+ * mask_token_id and becomes idle if the block held one of its n_stop stop_ids [bs, n_stop] (-1 = unused
+ * entry) or lens - first_len >= max_new, else denoising again.  status [bs, 4] int32 = (phase, lens,
+ * masked positions left, positions committed by this pass).
+ */
+int mdx_block_advance(int64_t* tokens, const uint8_t* transfer,
+                      int32_t* step_map, int32_t* step, int32_t* phase, int32_t* lens,
+                      const int32_t* first_len, const int32_t* max_new,
+                      const int64_t* stop_ids, int32_t n_stop,
+                      int64_t* out_tokens, int32_t* out_steps, int64_t out_stride,
+                      int32_t* status, int64_t mask_token_id,
+                      int32_t bs, int32_t block_len, mdx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -362,6 +362,85 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
     if (p == 0) count[b] = n_commit;
 }
 
+// The same rule for blocks of up to 64 positions (the engine's blocks hold 32) with ONE wavefront per
+// sequence: lane p owns position p, counts are ballots, and the rank among the masked positions comes
+// from reading every lane's confidence in turn -- no LDS, no atomics, no barrier, so the launch costs
+// little more than its one round trip to memory.
+template <bool FROM_PARTIALS>
+__global__ __launch_bounds__(mdx::kWave) void select_transfer_wave_kernel(
+    int64_t* __restrict__ x0, float* __restrict__ x0_p, int64_t* __restrict__ tokens,
+    const Partial* __restrict__ partials, int nsplit, const float* __restrict__ temperatures,
+    int64_t mask_token_id, float threshold, int k,
+    uint8_t* __restrict__ transfer, int32_t* __restrict__ count, int block_len)
+{
+    const int b = blockIdx.x;
+    const int p = threadIdx.x;
+    const bool on = p < block_len;
+    const int64_t at = (int64_t)b * block_len + p;
+    int64_t pick = 0;
+    float pick_p = 0.f;
+    int64_t tok = 0;
+    if (on) {
+        tok = tokens[at];
+        if (FROM_PARTIALS) {
+            const float c = kLog2e / (temperatures ? temperatures[b] : 1.0f);
+            Partial r = partials[at * nsplit];
+            for (int s = 1; s < nsplit; ++s) combine(r, partials[at * nsplit + s], c, false);
+            finish_row<false>(r, c, pick, pick_p);
+            x0[at] = pick;
+            x0_p[at] = pick_p;
+        } else {
+            pick = x0[at];
+            pick_p = x0_p[at];
+        }
+    }
+    const bool masked = on && tok == mask_token_id;
+    const float conf = masked ? pick_p : -INFINITY;
+    const bool hi = conf > threshold;
+    bool commit;
+    if (__popcll(__ballot(hi)) >= k) {
+        commit = hi;
+    } else {
+        // rank among masked positions: higher confidence first, lower position first on ties
+        int rank = 0;
+        for (int j = 0; j < block_len; ++j) {
+            const float cj = __shfl(conf, j);
+            rank += (cj > conf || (cj == conf && j < p)) ? 1 : 0;
+        }
+        commit = masked && rank < k;     // at most min(k, #masked) positions
+    }
+    const int n_commit = __popcll(__ballot(commit));
+    if (on) {
+        transfer[at] = commit ? 1 : 0;
+        if (commit) tokens[at] = pick;
+    }
+    if (p == 0) count[b] = n_commit;
+}
+
+int launch_select(int64_t* x0, float* x0_p, int64_t* tokens, const Partial* partials, int nsplit, const float* temperatures,
+                  int64_t mask_token_id, float threshold, int k, uint8_t* transfer, int32_t* count, int bs, int block_len,
+                  hipStream_t stream)
+{
+    const bool from_partials = partials != nullptr && nsplit > 1;
+    if (block_len <= mdx::kWave) {
+        if (from_partials)
+            select_transfer_wave_kernel<true><<<(unsigned)bs, mdx::kWave, 0, stream>>>(
+                x0, x0_p, tokens, partials, nsplit, temperatures, mask_token_id, threshold, k, transfer, count, block_len);
+        else
+            select_transfer_wave_kernel<false><<<(unsigned)bs, mdx::kWave, 0, stream>>>(
+                x0, x0_p, tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
+    } else {
+        const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
+        if (from_partials)
+            select_transfer_kernel<true><<<(unsigned)bs, threads, 0, stream>>>(
+                x0, x0_p, tokens, partials, nsplit, temperatures, mask_token_id, threshold, k, transfer, count, block_len);
+        else
+            select_transfer_kernel<false><<<(unsigned)bs, threads, 0, stream>>>(
+                x0, x0_p, tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
+    }
+    return mdx::check_launch("select_transfer");
+}
+
 // Splits per row so that small batches still fill the chip: target >= 4 workgroups per CU
 // while keeping at least 32 KiB of logits per workgroup.
 int pick_nsplit(int64_t rows, int64_t vocab) {
@@ -461,10 +540,8 @@ extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t
     MDX_REQUIRE(x0 && x0_p && tokens && transfer && count, MDX_EINVAL, "select_transfer: null pointer");
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "select_transfer: block_len %d > %d", block_len, kMaxBlockLen);
     MDX_REQUIRE(k >= 1, MDX_EINVAL, "select_transfer: k %d < 1", k);
-    const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
-    select_transfer_kernel<false><<<(unsigned)bs, threads, 0, stream>>>(
-        const_cast<int64_t*>(x0), const_cast<float*>(x0_p), tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
-    return mdx::check_launch("select_transfer");
+    return launch_select(const_cast<int64_t*>(x0), const_cast<float*>(x0_p), tokens, nullptr, 1, nullptr, mask_token_id, threshold, k,
+                         transfer, count, bs, block_len, stream);
 }
 
 extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
@@ -485,12 +562,6 @@ extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t d
     int rc = confidence_pass(logits, row_stride, dtype, temperatures, block_len, noise, noise_row_stride,
                              x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, noise != nullptr, &nsplit, stream);
     if (rc != MDX_OK) return rc;
-    const int threads = ((block_len + mdx::kWave - 1) / mdx::kWave) * mdx::kWave;
-    if (nsplit > 1 && !noise)
-        select_transfer_kernel<true><<<(unsigned)bs, threads, 0, stream>>>(
-            x0, x0_p, tokens, static_cast<const Partial*>(workspace), nsplit, temperatures, mask_token_id, threshold, k, transfer, count, block_len);
-    else
-        select_transfer_kernel<false><<<(unsigned)bs, threads, 0, stream>>>(
-            x0, x0_p, tokens, nullptr, 1, nullptr, mask_token_id, threshold, k, transfer, count, block_len);
-    return mdx::check_launch("select_transfer");
+    return launch_select(x0, x0_p, tokens, (nsplit > 1 && !noise) ? static_cast<const Partial*>(workspace) : nullptr, nsplit, temperatures,
+                         mask_token_id, threshold, k, transfer, count, bs, block_len, stream);
 }

@@ -29,6 +29,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from . import _lib
 from .context import get_context, reset_context, set_context
 from .layers import Attention
 from .ops import (confidence_argmax, flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
@@ -85,7 +86,6 @@ class Sequence:
         self.current_denoising_block = torch.full((denoising_block_size,), mask_token_id, dtype=torch.int64)
         self.current_step_map = torch.zeros((denoising_block_size,), dtype=torch.int32)
         self.current_denoise_step = 0
-        self.block_has_mask = None                       # filled by the engine's sampler; see postprocess
 
     def __len__(self):
         return self.num_tokens
@@ -301,23 +301,41 @@ class Decoder(nn.Module):
 
 
 # ----------------------------------------------------------------------------- engine
+IDLE, DENOISING, CACHING = 0, 1, 2      # MDX_PHASE_* of include/mdx.h: the per-lane state of the device loop
+N_STOP = 4                              # stop-token ids per sequence that the device loop can check
+
+
+class _PagesShort(Exception):
+    """The page pool cannot cover what the device loop wants ahead of a sequence."""
+
+
 class BlockDiffusionEngine:
-    """Scheduler + runner for block-diffusion decoding (llm_engine.py:66-73 `step`, scheduler.py,
-    model_runner.py:127-219), one GPU, eager."""
+    """Scheduler + runner for block-diffusion decoding on one GPU (llm_engine.py:66-73 `step`,
+    scheduler.py:24-82, model_runner.py:127-219).
+
+    Two decode paths share the same kernels:
+      * host-driven (decode_graphs=False, or a test hook is installed): every pass is prepared on the
+        host, run eagerly, and its results are downloaded -- the reference's own control flow;
+      * the device loop (decode_graphs=True): block tokens, lengths, step maps and the
+        denoise -> caching -> append state machine live on the device (csrc/block_state.hip); a pass is two
+        HIP-graph replays (decoder forward, then vocabulary projection + unmask step + state advance) with
+        no upload and no blocking download, and the host reads a 16-byte status per sequence one
+        pass late, while the next pass already runs."""
 
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
                  max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
                  decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True,
                  replay_ahead: bool = True, gumbel_seed: int | None = None):
         self.model = model
-        self.decode_graphs = decode_graphs                 # replay a captured HIP graph per decode batch size
+        self.decode_graphs = decode_graphs                 # decode through the device loop (HIP graphs per batch size)
         self.max_model_len = max_model_len
         # Gumbel noise on the scaled logits before the argmax, as Sampler.prepare draws it (sampler.py:15-18);
         # None = plain argmax (reproducible), an int seeds a device generator (reproducible per seed)
         self.gumbel = None if gumbel_seed is None else torch.Generator(device=model.lm_head.device).manual_seed(gumbel_seed)
-        self.replay_ahead = replay_ahead                   # graph decode: enqueue the next forward before the host bookkeeping
-        self.masked_rows_only = masked_rows_only           # graph decode: logits for still-masked positions only
-        self._graphs = {}
+        self.replay_ahead = replay_ahead                   # device loop: enqueue pass p+1 before reading the status of pass p
+        self.masked_rows_only = masked_rows_only           # device loop: logits for still-masked positions only
+        self._graphs = {}                                  # captured batch size -> lane buffers and graphs
+        self._loaded = None                                # the lanes that currently hold the running sequences
         self._temps = None
         self.c = model.c
         self.device = model.lm_head.device
@@ -337,7 +355,7 @@ class BlockDiffusionEngine:
             layer.attn.v_cache = self.kv_cache[1, i]
         self.stats = dict(prefill_passes=0, decode_passes=0, committed_tokens=0, prefill_s=0.0, decode_s=0.0)
 
-    # ---- requests / scheduling (scheduler.py:21-63) ----
+    # ---- requests / scheduling ----
     def add_request(self, token_ids, sampling_params=None, prefix_embeds=None) -> Sequence:
         seq = Sequence(token_ids, sampling_params, self.c.block_size, self.c.mask_token_id, prefix_embeds)
         self.waiting.append(seq)
@@ -346,37 +364,50 @@ class BlockDiffusionEngine:
     def is_finished(self):
         return not self.waiting and not self.running
 
-    def schedule(self):
-        scheduled, tokens = [], 0
-        while self.waiting and len(scheduled) < self.max_num_seqs:
+    def _admit(self):
+        """The prefill batch: requests from the head of the waiting queue, in arrival order, while the
+        token budget, the sequence limit and the page pool allow (scheduler.py:24-42)."""
+        batch, tokens = [], 0
+        while self.waiting and len(batch) < self.max_num_seqs:
             seq = self.waiting[0]
             if tokens + len(seq) > self.max_num_batched_tokens or not self.block_manager.can_allocate(seq):
                 break
             self.block_manager.allocate(seq)
             tokens += len(seq)
             seq.status = SequenceStatus.RUNNING
-            self.waiting.popleft()
-            self.running.append(seq)
-            scheduled.append(seq)
-        if scheduled:
-            return scheduled, True
-        # decode (scheduler.py:44-58): a sequence that cannot get the page its next block needs makes
-        # room by preempting the sequence at the back of the queue (or itself, when it is alone)
-        while self.running and len(scheduled) < self.max_num_seqs:
+            self.running.append(self.waiting.popleft())
+            batch.append(seq)
+        return batch
+
+    def _grow(self):
+        """The decode batch of a host-driven pass: every running sequence gets the page its block needs; when
+        the pool is empty, the sequence at the back of the queue gives its pages up (or, alone, the
+        sequence itself) and goes back to the waiting queue (scheduler.py:44-63)."""
+        batch = []
+        while self.running and len(batch) < self.max_num_seqs:
             seq = self.running.popleft()
+            evicted_itself = False
             while not self.block_manager.can_append(seq):
                 if self.running:
                     self.preempt(self.running.pop())
                 else:
                     self.preempt(seq)
+                    evicted_itself = True
                     break
-            else:
+            if not evicted_itself:
                 self.block_manager.may_append(seq)
-                scheduled.append(seq)
-        if not scheduled:
+                batch.append(seq)
+        if not batch:
             raise RuntimeError("KV pool too small for a single sequence")
-        self.running.extendleft(reversed(scheduled))
-        return scheduled, False
+        self.running.extendleft(reversed(batch))
+        return batch
+
+    def schedule(self):
+        """(sequences, is_prefill) of the next host-driven pass: prefill first (scheduler.py:24-58)."""
+        batch = self._admit()
+        if batch:
+            return batch, True
+        return self._grow(), False
 
     def preempt(self, seq):                                # scheduler.py:60-63: back to the queue, its pages freed;
         seq.status = SequenceStatus.WAITING                # the next prefill recomputes its cache (the block in
@@ -384,28 +415,29 @@ class BlockDiffusionEngine:
         self.waiting.appendleft(seq)
         self.stats["preemptions"] = self.stats.get("preemptions", 0) + 1
 
-    def postprocess(self, seqs):                           # scheduler.py:65-82
+    def postprocess(self, seqs):
+        """After a host-driven pass (scheduler.py:65-82): a sequence whose block has no mask left is due
+        for its caching pass; one that just had it appends the block and either ends or starts a new one."""
         for seq in seqs:
-            if not seq.is_caching:
-                probe = seq.block_has_mask                  # (block tensor, any mask left) noted by `sample`
-                if probe is not None and probe[0] is seq.current_denoising_block:
-                    masked = probe[1]
-                else:
-                    masked = bool((seq.current_denoising_block == seq.mask_token_id).any())
-                if not masked:
+            if seq.status != SequenceStatus.CACHING:
+                if not bool((seq.current_denoising_block == seq.mask_token_id).any()):
                     seq.status = SequenceStatus.CACHING
                 continue
-            finished = any((seq.current_denoising_block == s).any() for s in seq.sampling_params.stop_token_ids)
+            block = seq.current_denoising_block
+            stopped = any(bool((block == s).any()) for s in seq.sampling_params.stop_token_ids)
             seq.append_block()
             self.stats["committed_tokens"] += seq.denoising_block_size
-            if (not seq.ignore_eos and finished) or seq.num_completion_tokens >= seq.max_new_tokens:
-                seq.status = SequenceStatus.FINISHED
-                self.block_manager.deallocate(seq)
-                self.running.remove(seq)
+            if (stopped and not seq.ignore_eos) or seq.num_completion_tokens >= seq.max_new_tokens:
+                self._retire(seq)
             else:
                 seq.status = SequenceStatus.RUNNING
 
-    # ---- runner (model_runner.py:121-219) ----
+    def _retire(self, seq):
+        seq.status = SequenceStatus.FINISHED
+        self.block_manager.deallocate(seq)
+        self.running.remove(seq)
+
+    # ---- host-driven runner (model_runner.py:121-219) ----
     def _block_tables(self, seqs):
         n = max(len(s.block_table) for s in seqs)
         bt = torch.full((len(seqs), n), -1, dtype=torch.int32)
@@ -453,95 +485,6 @@ class BlockDiffusionEngine:
                     block_tables=self._block_tables(seqs), block_size=S)
         return ids.to(dev, non_blocking=True), pos.to(dev, non_blocking=True)
 
-    # ---- decode graphs (model_runner.py:198-211 replay, :221-259 capture) ----
-    def _capture_decode(self, bs: int):
-        """Static input buffers + one captured forward of the decoder for `bs` sequences.  Every libmdx
-        launch goes to torch's current stream and allocates nothing itself, so the capture records
-        them like any torch op; page tables have their maximum width so that the split-KV launch
-        geometry is the same for every replay.  The five inputs are views into one device buffer
-        that mirrors one pinned host buffer: a pass uploads them with a single copy."""
-        S, dev = self.c.block_size, self.device
-        width = (self.max_model_len + PAGE - 1) // PAGE
-        fields = [("ids", torch.int64, (bs, S)), ("pos", torch.int64, (bs, S)), ("slots", torch.int32, (bs, S)),
-                  ("lens", torch.int32, (bs,)), ("bt", torch.int32, (bs, width))]
-        offsets, at = {}, 0
-        for name, dt, shape in fields:
-            offsets[name] = at
-            at += (math.prod(shape) * dt.itemsize + 15) // 16 * 16
-        g = dict(dev_buf=torch.zeros(at, dtype=torch.uint8, device=dev),
-                 pin_buf=torch.zeros(at, dtype=torch.uint8, pin_memory=True), host={})
-        for name, dt, shape in fields:
-            n = math.prod(shape) * dt.itemsize
-            g[name] = g["dev_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
-            g["host"][name] = g["pin_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
-        g["host"]["slots"].fill_(-1)
-        g["host"]["bt"].fill_(-1)
-        g["dev_buf"].copy_(g["pin_buf"])
-        g["result"] = torch.zeros(2, bs, S, dtype=torch.int64, device=dev)          # tokens, transfer flags
-        g["result_host"] = torch.zeros(2, bs, S, dtype=torch.int64, pin_memory=True)
-        g["downloaded"] = torch.cuda.Event()
-        g["idx_host"] = torch.zeros(bs * S, dtype=torch.int64, pin_memory=True)       # rows still masked
-        g["idx_dev"] = torch.zeros(bs * S, dtype=torch.int64, device=dev)
-        set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):                      # warm-up outside the capture (library handles, autotuning)
-            self.model(self.model.embed(g["ids"]), g["pos"])
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        g["graph"] = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g["graph"], stream=side):    # the stream of the warm-up: its per-stream buffers exist
-            g["hidden"] = self.model(self.model.embed(g["ids"]), g["pos"])
-        torch.cuda.synchronize()
-        return g
-
-    def _graph_batch(self, bs: int) -> int:
-        """The captured batch size that serves `bs` sequences: 1, 2, 4, 8, then multiples of 16
-        (model_runner.py:233,200); the rows in excess are padding (slot -1, context length 0)."""
-        for b in (1, 2, 4, 8):
-            if bs <= b:
-                return b
-        return (bs + 15) // 16 * 16
-
-    def _run_decode_graph(self, seqs):
-        """Uploads the pass inputs (one copy) and replays the graph.  Within a denoising block
-        nothing has to be uploaded at all: lengths, slots and page tables are those of the previous
-        pass, and the token block on the device is the one the unmask step just updated in place
-        (the host rows handed to the sequences by `sample` are a download of exactly that buffer)."""
-        S, bs = self.c.block_size, len(seqs)
-        gbs = self._graph_batch(bs)
-        g = self._graphs.get(gbs)
-        if g is None:
-            g = self._graphs[gbs] = self._capture_decode(gbs)
-        signature = [(s.seq_id, s.num_tokens, len(s.block_table)) for s in seqs]
-        rows = g.get("rows")
-        fresh = (g.get("signature") == signature and rows is not None
-                 and all(s.current_denoising_block is r for s, r in zip(seqs, rows)))
-        if not fresh:
-            h = g["host"]
-            torch.stack([s.current_denoising_block for s in seqs], out=h["ids"][:bs])
-            lens = torch.tensor([len(s) for s in seqs], dtype=torch.int64)
-            torch.add(lens.unsqueeze(1), torch.arange(S), out=h["pos"][:bs])
-            h["slots"].fill_(-1)                            # padding rows: nothing stored, no context (model_runner.py:203-206)
-            h["slots"][:bs] = torch.tensor([s.get_slots(len(s), len(s) + S) for s in seqs], dtype=torch.int32)
-            h["lens"].zero_()
-            h["lens"][:bs] = lens + S
-            h["ids"][bs:] = 0
-            h["pos"][bs:] = 0
-            h["bt"].fill_(-1)
-            for i, s in enumerate(seqs):
-                h["bt"][i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
-            g["dev_buf"].copy_(g["pin_buf"], non_blocking=True)
-            g["signature"] = signature
-            g["x_host"] = h["ids"][:bs]                     # host copy of the device token blocks
-        set_context(False, slot_mapping=g["slots"], context_lens=g["lens"], block_tables=g["bt"], block_size=S)
-        ahead = g.pop("replayed_ahead", False)              # enqueued by the previous pass's `_download`?
-        for other in self._graphs.values():
-            other.pop("replayed_ahead", None)               # a forward enqueued ahead for another batch is void
-        if not (fresh and ahead):
-            g["graph"].replay()
-        return g["hidden"], g
-
     def _noise(self, logits):
         if self.gumbel is None:
             return None
@@ -554,131 +497,352 @@ class BlockDiffusionEngine:
             self._temps = (key, torch.tensor(key, dtype=torch.float32, device=self.device))
         return self._temps[1]
 
-    def sample(self, logits, seqs, g=None) -> int:         # layers/sampler.py:24-61 on the device
-        """Unmask step on the device, then one download of (tokens, transfer flags).  With the
-        buffers `g` of a decode graph, the token block is the graph's own input buffer (already
-        on the device) and the download goes through one pinned buffer."""
+    def sample(self, logits, seqs) -> int:                 # layers/sampler.py:24-61, selection on the device
         sp = seqs[0].sampling_params
         if sp.denoising_strategy != "low_confidence_dynamic":
             raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
-        if g is not None:
-            x = g["ids"][:len(seqs)]
-        else:
-            x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
+        x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
         extra = {} if self.gumbel is None else {"noise": self._noise(logits)}
         _, _, transfer, _n = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
                                          temperatures=self._temperatures(seqs), **extra)
-        if g is None:
-            x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
-            for i, s in enumerate(seqs):
-                s.current_denoising_block = x_cpu[i]
-                s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
-                s.current_denoise_step += 1
-            return int(transfer_cpu.sum().item())
-        return self._download(seqs, g, x, transfer)
-
-    def _download(self, seqs, g, x, transfer) -> int:
-        """One download of (tokens, transfer flags) through the pinned buffer, then the per-sequence
-        bookkeeping of sampler.py:56-59 as batch operations."""
-        bs = len(seqs)
-        g["result"][0, :bs].copy_(x)
-        g["result"][1, :bs].copy_(transfer)
-        g["result_host"].copy_(g["result"], non_blocking=True)
-        g["downloaded"].record()
-        # The next pass's forward needs nothing from the host when no sequence of this pass is about
-        # to append its block (then lengths, slots and page tables stay, and the token block is on
-        # the device already): enqueue it now, so that the GPU runs it while the host does the
-        # bookkeeping below.  `_run_decode_graph` checks that this really was the next pass.
-        if self.replay_ahead and not any(s.is_caching for s in seqs):
-            g["graph"].replay()
-            g["replayed_ahead"] = True
-        g["downloaded"].synchronize()
-        x_cpu, transfer_cpu = g["result_host"][0, :bs].clone(), g["result_host"][1, :bs].bool()
-        g["x_host"] = x_cpu
-        # one indexed write for all step maps: the sequences' maps are rows of one batch tensor
-        maps, map_rows = g.get("maps"), g.get("map_rows")
-        if maps is None or not all(s.current_step_map is r for s, r in zip(seqs, map_rows)):
-            maps = g["maps"] = torch.stack([s.current_step_map for s in seqs])
-            map_rows = g["map_rows"] = list(maps.unbind(0))
-            for s, r in zip(seqs, map_rows):
-                s.current_step_map = r
-        steps = torch.tensor([s.current_denoise_step for s in seqs], dtype=torch.int32)
-        maps[transfer_cpu] = steps.unsqueeze(1).expand_as(maps)[transfer_cpu]
-        rows = g["rows"] = list(x_cpu.unbind(0))
-        has_mask = (x_cpu == seqs[0].mask_token_id).any(1).tolist()
-        for s, r, m in zip(seqs, rows, has_mask):
-            s.current_denoising_block = r
-            s.block_has_mask = (r, m)
+        x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
+        for i, s in enumerate(seqs):
+            s.current_denoising_block = x_cpu[i]
+            s.current_step_map[transfer_cpu[i]] = s.current_denoise_step
             s.current_denoise_step += 1
         return int(transfer_cpu.sum().item())
 
-    def _sample_masked_rows(self, hidden, seqs, g) -> int:
-        """The unmask step restricted to the positions that are still masked.  The selection reads
-        confidences of masked positions only (sampler.py:39) and commits x0 only there (:54), so the
-        logits of committed positions are never looked at: the vocabulary projection, the softmax
-        and the argmax run on the masked rows alone (half the rows on average, none in the pass
-        that only caches a finished block), with identical results."""
-        sp = seqs[0].sampling_params
-        if sp.denoising_strategy != "low_confidence_dynamic":
-            raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
-        S, bs, mask_id = self.c.block_size, len(seqs), seqs[0].mask_token_id
-        idx = (g["x_host"].reshape(-1) == mask_id).nonzero().squeeze(1)
-        if idx.numel() == 0:
-            for s in seqs:
-                s.current_denoise_step += 1
-            return 0
-        # through pinned memory: a copy from pageable memory would hold the host until the stream,
-        # which may already hold the next forward, has drained
-        n = idx.numel()
-        g["idx_host"][:n].copy_(idx)
-        idx_dev = g["idx_dev"][:n]
-        idx_dev.copy_(g["idx_host"][:n], non_blocking=True)
-        logits = F.linear(hidden.flatten(0, 1).index_select(0, idx_dev), self.model.lm_head)   # rows of the first bs sequences
-        temps = self._temperatures(seqs)
-        if len(set(self._temps[0])) == 1:
-            temps = temps[:1]
-        else:
-            temps = temps.index_select(0, idx_dev // S)
-        x0_rows, p_rows = confidence_argmax(logits, temps, self._noise(logits))
-        if "x0" not in g:
-            g["x0"] = torch.zeros(g["ids"].numel(), dtype=torch.int64, device=self.device)
-            g["x0_p"] = torch.zeros(g["ids"].numel(), dtype=torch.float32, device=self.device)
-        g["x0"].index_copy_(0, idx_dev, x0_rows)
-        g["x0_p"].index_copy_(0, idx_dev, p_rows)
-        transfer, _n = select_transfer(g["x0"][:bs * S].view(bs, S), g["x0_p"][:bs * S].view(bs, S), g["ids"][:bs], mask_id,
-                                       sp.dynamic_threshold, sp.transfer_count)
-        return self._download(seqs, g, g["ids"][:bs], transfer)
-
     @torch.inference_mode()
-    def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219
-        if not is_prefill and self.decode_graphs and max(len(s) for s in seqs) + self.c.block_size <= self.max_model_len:
-            hidden, g = self._run_decode_graph(seqs)
-        else:
-            g = None
-            ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
-            hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
-        if g is not None and self.masked_rows_only and self.on_logits is None and self.unmask is unmask_step:
-            n = self._sample_masked_rows(hidden, seqs, g)
-            reset_context()
-            return n
-        logits = self.model.compute_logits(hidden if g is None else hidden[:len(seqs)])
+    def run(self, seqs, is_prefill: bool) -> int:          # model_runner.py:213-219, host-driven
+        ids, pos = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+        hidden = self.model(self._embed(seqs, ids, is_prefill), pos)
+        logits = self.model.compute_logits(hidden)
         if is_prefill:
             logits = logits.view(len(seqs), self.c.block_size, -1)
         if self.on_logits is not None:
             self.on_logits(is_prefill, seqs, logits)
-        n = self.sample(logits, seqs, g)
+        n = self.sample(logits, seqs)
         reset_context()
         return n
 
+    # ---- the device loop ----------------------------------------------------------------------------------
+    def _graph_batch(self, bs: int) -> int:
+        """The captured batch size that serves `bs` sequences: 1, 2, 4, 8, then multiples of 16
+        (model_runner.py:233,200); the lanes in excess are idle (slot -1, context length 0)."""
+        for b in (1, 2, 4, 8):
+            if bs <= b:
+                return b
+        return (bs + 15) // 16 * 16
+
+    def _device_loop_usable(self, seqs) -> bool:
+        if not self.decode_graphs or self.on_logits is not None or self.unmask is not unmask_step:
+            return False
+        sp = seqs[0].sampling_params
+        if sp.denoising_strategy != "low_confidence_dynamic":
+            raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
+        S = self.c.block_size
+        return all(s.num_prompt_tokens + -(-s.max_new_tokens // S) * S + S <= self.max_model_len and
+                   len(s.sampling_params.stop_token_ids) <= N_STOP for s in seqs)
+
+    def _make_lanes(self, gbs: int):
+        """Static buffers of the lanes of one captured batch size and the graph of the decoder forward over them.
+        The state a (re)load writes is one device buffer mirrored by one pinned host buffer (a single copy)."""
+        S, dev = self.c.block_size, self.device
+        width = (self.max_model_len + PAGE - 1) // PAGE
+        i32, i64, f32 = torch.int32, torch.int64, torch.float32
+        fields = [("ids", i64, (gbs, S)), ("stop_ids", i64, (gbs, N_STOP)), ("step_map", i32, (gbs, S)), ("lens", i32, (gbs,)),
+                  ("phase", i32, (gbs,)), ("step", i32, (gbs,)), ("first_len", i32, (gbs,)), ("max_new", i32, (gbs,)),
+                  ("temps", f32, (gbs,)), ("bt", i32, (gbs, width))]
+        offsets, at = {}, 0
+        for name, dt, shape in fields:
+            offsets[name] = at
+            at += (math.prod(shape) * dt.itemsize + 15) // 16 * 16
+        g = dict(bs=gbs, width=width, dev_buf=torch.zeros(at, dtype=torch.uint8, device=dev),
+                 pin_buf=torch.zeros(at, dtype=torch.uint8, pin_memory=True), host={}, heads={}, pass_no=0)
+        for name, dt, shape in fields:
+            n = math.prod(shape) * dt.itemsize
+            g[name] = g["dev_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
+            g["host"][name] = g["pin_buf"][offsets[name]:offsets[name] + n].view(dt).view(shape)
+        g["pos"] = torch.zeros(gbs, S, dtype=i64, device=dev)                  # written by mdx_block_prepare every pass
+        g["slots"] = torch.full((gbs, S), -1, dtype=i32, device=dev)
+        g["ctx"] = torch.zeros(gbs, dtype=i32, device=dev)
+        g["x0"] = torch.zeros(gbs * S, dtype=i64, device=dev)
+        g["x0_p"] = torch.zeros(gbs * S, dtype=f32, device=dev)
+        g["rows"] = torch.zeros(gbs * S, dtype=i64, device=dev)
+        g["n_rows"] = torch.zeros(1, dtype=i32, device=dev)
+        g["out_tokens"] = torch.zeros(gbs, self.max_model_len, dtype=i64, device=dev)
+        g["out_steps"] = torch.zeros(gbs, self.max_model_len, dtype=i32, device=dev)
+        g["status"] = torch.zeros(gbs, 4, dtype=i32, device=dev)
+        g["status_host"] = torch.zeros(2, gbs, 4, dtype=i32, pin_memory=True)
+        g["status_done"] = [torch.cuda.Event(), torch.cuda.Event()]
+        g["bt_copied"] = torch.cuda.Event()
+        g["host"]["bt"].fill_(-1)
+        g["host"]["stop_ids"].fill_(-1)
+        g["host"]["temps"].fill_(1.0)
+        g["dev_buf"].copy_(g["pin_buf"])
+        side = torch.cuda.Stream()
+        g["stream"] = side
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                      # warm-up outside the capture (library handles, autotuning)
+            self._forward_lanes(g)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g["fwd"] = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g["fwd"], stream=side):      # the stream of the warm-up: its per-stream buffers exist
+            g["hidden"] = self._forward_lanes(g)
+        torch.cuda.synchronize()
+        return g
+
+    def _forward_lanes(self, g):
+        """prepare_decode on the device (positions, slots, context lengths from the lanes' lengths and page
+        tables), then the decoder forward over the lanes' blocks."""
+        S = self.c.block_size
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(_lib.lib().mdx_block_prepare(g["lens"].data_ptr(), g["phase"].data_ptr(), g["bt"].data_ptr(), g["bt"].stride(0),
+                                                g["width"], PAGE, S, g["pos"].data_ptr(), g["slots"].data_ptr(), g["ctx"].data_ptr(),
+                                                g["bs"], stream), "block_prepare")
+        set_context(False, slot_mapping=g["slots"], context_lens=g["ctx"], block_tables=g["bt"], block_size=S)
+        hidden = self.model(self.model.embed(g["ids"]), g["pos"])
+        reset_context()
+        return hidden
+
+    def _logits_of_rows(self, g, cap: int):
+        """Vocabulary projection + confidence / argmax on `cap` rows: the still-masked ones compacted on the device
+        (cap < all rows), or all of them.  Results land in the lanes' x0 / x0_p."""
+        S, gbs = self.c.block_size, g["bs"]
+        flat = g["hidden"].flatten(0, 1)
+        if cap < gbs * S:
+            rows = g["rows"][:cap]
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            _lib.check(_lib.lib().mdx_masked_rows(g["ids"].data_ptr(), g["phase"].data_ptr(), self.c.mask_token_id, gbs, S,
+                                                  rows.data_ptr(), cap, g["n_rows"].data_ptr(), stream), "masked_rows")
+            logits = F.linear(flat.index_select(0, rows), self.model.lm_head)
+            x0, p = confidence_argmax(logits, g["temps"].index_select(0, rows // S), self._noise(logits))
+            g["x0"].index_copy_(0, rows, x0)
+            g["x0_p"].index_copy_(0, rows, p)
+        else:
+            logits = F.linear(flat, self.model.lm_head).view(gbs, S, -1)
+            x0, p = confidence_argmax(logits, g["temps"], self._noise(logits))
+            g["x0"].copy_(x0.view(-1))
+            g["x0_p"].copy_(p.view(-1))
+
+    def _head(self, g, cap: int, threshold: float, k: int):
+        """The second half of a pass: logits of (at most) `cap` masked rows, the selection rule, and the advance of
+        every lane's state (sampler.py:24-61 + scheduler.py:65-82 on the device)."""
+        S, gbs = self.c.block_size, g["bs"]
+        if cap > 0:
+            self._logits_of_rows(g, cap)
+        transfer, _count = select_transfer(g["x0"].view(gbs, S), g["x0_p"].view(gbs, S), g["ids"], self.c.mask_token_id, threshold, k)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(_lib.lib().mdx_block_advance(
+            g["ids"].data_ptr(), transfer.data_ptr(), g["step_map"].data_ptr(), g["step"].data_ptr(), g["phase"].data_ptr(),
+            g["lens"].data_ptr(), g["first_len"].data_ptr(), g["max_new"].data_ptr(), g["stop_ids"].data_ptr(), N_STOP,
+            g["out_tokens"].data_ptr(), g["out_steps"].data_ptr(), g["out_tokens"].stride(0), g["status"].data_ptr(),
+            self.c.mask_token_id, gbs, S, stream), "block_advance")
+
+    def _head_graph(self, g, cap, threshold, k):
+        key = (cap, threshold, k)
+        graph = g["heads"].get(key)
+        if graph is None:
+            outer = torch.cuda.current_stream()
+            g["stream"].wait_stream(outer)
+            with torch.cuda.stream(g["stream"]):           # warm the projection at this row count; touches scratch only, no lane state
+                if cap > 0:
+                    self._logits_of_rows(g, cap)
+            outer.wait_stream(g["stream"])
+            torch.cuda.synchronize()
+            if "head_pool" not in g:                        # the variants hold temporaries only and never run together: one pool
+                g["head_pool"] = torch.cuda.graph_pool_handle()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=g["head_pool"], stream=g["stream"]):
+                self._head(g, cap, threshold, k)
+            torch.cuda.synchronize()
+            g["heads"][key] = graph
+        return graph
+
+    def _load_lanes(self, seqs):
+        """Puts the state of `seqs` (as the host knows it) into the lanes of the batch size that serves them."""
+        S, mask = self.c.block_size, self.c.mask_token_id
+        gbs = self._graph_batch(len(seqs))
+        g = self._graphs.get(gbs)
+        if g is None:
+            g = self._graphs[gbs] = self._make_lanes(gbs)
+        g["bt_copied"].synchronize()
+        h = g["host"]
+        h["phase"].zero_()
+        h["lens"].zero_()
+        h["bt"].fill_(-1)
+        h["stop_ids"].fill_(-1)
+        h["ids"].fill_(mask)
+        for i, s in enumerate(seqs):
+            h["ids"][i] = s.current_denoising_block
+            h["step_map"][i] = s.current_step_map
+            h["lens"][i] = len(s)
+            h["phase"][i] = CACHING if s.status == SequenceStatus.CACHING else DENOISING
+            h["step"][i] = s.current_denoise_step
+            h["first_len"][i] = s.num_prompt_tokens
+            h["max_new"][i] = s.max_new_tokens
+            h["temps"][i] = s.temperature
+            stops = [] if s.ignore_eos else list(s.sampling_params.stop_token_ids)
+            h["stop_ids"][i, :len(stops)] = torch.tensor(stops, dtype=torch.int64)
+            h["bt"][i, :len(s.block_table)] = torch.tensor(s.block_table, dtype=torch.int32)
+        g["dev_buf"].copy_(g["pin_buf"], non_blocking=True)
+        g["bt_copied"].record()
+        masked = (h["ids"][:len(seqs)] == mask).sum(1).tolist()
+        g["seqs"] = list(seqs)
+        g["known"] = dict(at_pass=g["pass_no"], phase=h["phase"][:len(seqs)].tolist(), masked=masked, lens=h["lens"][:len(seqs)].tolist())
+        g["live_at"] = {}                                   # pass number -> lanes that were live at its start, as far as known
+        g["pending"] = []                                   # passes enqueued whose status has not been read yet
+        self._loaded = g
+        return g
+
+    def _cover_pages(self, g):
+        """Every live lane's page table must reach as far as the device can get before the host next looks:
+        the block being denoised, the block after it, and one more block for the pass in flight."""
+        S = self.c.block_size
+        changed = False
+        for i, s in enumerate(g["seqs"]):
+            if g["known"]["phase"][i] == IDLE:
+                continue
+            last = min(g["known"]["lens"][i] + 3 * S, s.num_prompt_tokens + -(-s.max_new_tokens // S) * S)
+            want = (last + PAGE - 1) // PAGE
+            while len(s.block_table) < want:
+                if not self.block_manager.free:
+                    raise _PagesShort()
+                if not changed:
+                    g["bt_copied"].synchronize()             # the previous upload of the tables has left the pinned buffer
+                    changed = True
+                g["host"]["bt"][i, len(s.block_table)] = self.block_manager.free[0]
+                s.block_table.append(self.block_manager.free.popleft())
+        if changed:
+            g["bt"].copy_(g["host"]["bt"], non_blocking=True)
+            g["bt_copied"].record()
+
+    def _rows_cap(self, g) -> int:
+        """An upper bound, known without asking the device, of the masked rows at the start of the pass about to be
+        enqueued, rounded up to an eighth of all rows: every denoising pass commits at least min(k, masked)
+        positions of a lane, a caching pass leaves a fresh block behind."""
+        S, gbs = self.c.block_size, g["bs"]
+        if not self.masked_rows_only:
+            return gbs * S
+        kn, k = g["known"], g["seqs"][0].sampling_params.transfer_count
+        ahead = g["pass_no"] - kn["at_pass"]
+        bound = 0
+        for ph, m in zip(kn["phase"], kn["masked"]):
+            if ahead == 0:
+                bound += m if ph == DENOISING else 0
+            else:
+                bound += S if ph == CACHING else max(0, m - k) if ph == DENOISING else 0
+        step = max(1, gbs * S // 8)
+        return min(gbs * S, -(-bound // step) * step)
+
+    def _read_status(self, g, pass_no):
+        """Takes in the status that pass `pass_no` left: lengths, phases and masked counts of the lanes."""
+        slot = pass_no % 2
+        g["status_done"][slot].synchronize()
+        st = g["status_host"][slot][:len(g["seqs"])].tolist()
+        kn = g["known"]
+        live_before = [ph != IDLE for ph in kn["phase"]]
+        moved = 0
+        for i, (ph, ln, masked, n_moved) in enumerate(st):
+            if not live_before[i]:
+                continue
+            kn["phase"][i], kn["lens"][i], kn["masked"][i] = ph, ln, masked
+            moved += n_moved
+        kn["at_pass"] = pass_no + 1
+        if any(live_before):
+            self.stats["decode_passes"] += 1
+        return moved, any(kn["phase"][i] == IDLE and live_before[i] for i in range(len(st)))
+
+    def _drain(self):
+        """Waits for the device loop, brings every loaded sequence's state back to the host and retires the finished ones."""
+        g = self._loaded
+        if g is None:
+            return
+        moved = 0
+        for pass_no in g["pending"]:
+            moved += self._read_status(g, pass_no)[0]
+        g["pending"] = []
+        torch.cuda.synchronize()
+        n = len(g["seqs"])
+        ids, step_map, step, lens = g["ids"][:n].cpu(), g["step_map"][:n].cpu(), g["step"][:n].tolist(), g["lens"][:n].tolist()
+        phase = g["phase"][:n].tolist()
+        for i, s in enumerate(g["seqs"]):
+            have = s.num_tokens - s.num_prompt_tokens
+            new = lens[i] - s.num_tokens
+            if new > 0:
+                s.token_ids.extend(g["out_tokens"][i, have:have + new].tolist())
+                s.step_map.extend(g["out_steps"][i, have:have + new].tolist())
+                s.num_tokens = lens[i]
+                self.stats["committed_tokens"] += new
+            s.current_denoising_block = ids[i].clone()
+            s.current_step_map = step_map[i].clone()
+            s.current_denoise_step = step[i]
+            if phase[i] == IDLE:
+                self._retire(s)
+            else:
+                s.status = SequenceStatus.CACHING if phase[i] == CACHING else SequenceStatus.RUNNING
+        self._loaded = None
+        return moved
+
+    @torch.inference_mode()
+    def _device_pass(self, seqs) -> int:
+        """Enqueues one decode pass of the device loop and, one pass late, looks at what the passes before it did."""
+        g = self._loaded
+        if g is None or g["seqs"] != seqs:
+            self._drain()
+            g = self._load_lanes(seqs)
+        self._cover_pages(g)
+        sp = seqs[0].sampling_params
+        cap = self._rows_cap(g)
+        if self.gumbel is None:
+            head = self._head_graph(g, cap, float(sp.dynamic_threshold), int(sp.transfer_count))
+            g["fwd"].replay()
+            head.replay()
+        else:                                               # the noise comes from a generator: drawn eagerly, pass by pass
+            g["fwd"].replay()
+            self._head(g, cap, float(sp.dynamic_threshold), int(sp.transfer_count))
+        slot = g["pass_no"] % 2
+        g["status_host"][slot].copy_(g["status"], non_blocking=True)
+        g["status_done"][slot].record()
+        g["pending"].append(g["pass_no"])
+        g["pass_no"] += 1
+        moved, finished = 0, False
+        keep = 1 if self.replay_ahead else 0               # passes that may stay unread while the next one is prepared
+        while len(g["pending"]) > keep:
+            n, fin = self._read_status(g, g["pending"].pop(0))
+            moved += n
+            finished |= fin
+        if finished:
+            self._drain()
+        return moved
+
     def step(self):                                        # llm_engine.py:66-73
-        seqs, is_prefill = self.schedule()
         t0 = time.perf_counter()
-        n = self.run(seqs, is_prefill)
-        self.postprocess(seqs)
-        dt = time.perf_counter() - t0
-        self.stats["prefill_passes" if is_prefill else "decode_passes"] += 1
-        self.stats["prefill_s" if is_prefill else "decode_s"] += dt
-        return n, is_prefill
+        batch = self._admit() if self.waiting else []
+        if batch:
+            self._drain()
+            n = self.run(batch, True)
+            self.postprocess(batch)
+            self.stats["prefill_passes"] += 1
+            self.stats["prefill_s"] += time.perf_counter() - t0
+            return n, True
+        seqs = list(self.running)[:self.max_num_seqs]
+        n = None
+        if self._device_loop_usable(seqs):
+            try:
+                n = self._device_pass(seqs)
+            except _PagesShort:
+                self._drain()                               # the host-driven pass below needs less ahead and may preempt
+        else:
+            self._drain()
+        if n is None:
+            seqs = self._grow()
+            n = self.run(seqs, False)
+            self.postprocess(seqs)
+            self.stats["decode_passes"] += 1
+        self.stats["decode_s"] += time.perf_counter() - t0
+        return n, False
 
     def generate(self):
         """Runs every queued request to completion; returns them in arrival order."""

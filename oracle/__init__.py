@@ -35,6 +35,11 @@ add_rms_norm                residual is the rounded sum; reduces to rms_norm_ref
                             F.rms_norm of the fp32 sum; variance taken before the rounding (a case
                             where the two differ)
 silu_and_mul                F.silu * other half; silu(0) = 0, silu(x) -> x and -> 0 in the tails
+block_prepare               get_slots (brute-force slot formula) per position; idle lanes = graph padding
+masked_rows                 numpy nonzero of the same mask
+block_advance               driven with select_transfer over whole generations: pass count = the closed form
+                            expected_passes, tokens / step maps / finish conditions equal to the host
+                            engine's Sequence + postprocess (an independent implementation), stop tokens
 dense_forward               built from the pinned attention oracle and plain matmuls; its mask
                             and SDPA are the functions above
 ==========================  =====================================================
@@ -52,5 +57,5 @@ from .staircase import (  # noqa: F401
 from .kvstore import store_kvcache  # noqa: F401
 from .unmask import confidence_argmax, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
 from .slots import slot_of, get_slots  # noqa: F401
-from .engine import dense_forward, expected_passes  # noqa: F401
+from .engine import dense_forward, expected_passes, block_prepare, masked_rows, block_advance  # noqa: F401
 from .fused import qk_norm_rope, rms_norm_ref, rope_ref, add_rms_norm, silu_and_mul  # noqa: F401

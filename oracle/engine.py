@@ -65,3 +65,74 @@ def expected_passes(block_len: int, k: int, n_blocks: int) -> int:
     takes ceil(block_len / k) denoising passes plus one pass that stores the committed block
     (engines/nano_dvlm/nanovllm/engine/scheduler.py:65-82)."""
     return n_blocks * (-(-block_len // k) + 1)
+
+
+# ---- per-lane block state (the device loop's three small kernels) -----------------------------------------
+IDLE, DENOISING, CACHING = 0, 1, 2
+
+
+def block_prepare(lens, phase, block_table, page: int, block_len: int):
+    """ModelRunner.prepare_decode (engines/nano_dvlm/nanovllm/engine/model_runner.py:169-185) per lane:
+    positions = len .. len + S - 1, slots through the page table (engine/sequence.py:117-141),
+    context length len + S; idle lanes are graph padding (model_runner.py:203-208): slots -1, context 0."""
+    lens, phase, bt = np.asarray(lens), np.asarray(phase), np.asarray(block_table)
+    bs = len(lens)
+    pos = np.zeros((bs, block_len), dtype=np.int64)
+    slots = np.full((bs, block_len), -1, dtype=np.int32)
+    ctx = np.zeros(bs, dtype=np.int32)
+    for b in range(bs):
+        if phase[b] == IDLE:
+            continue
+        ctx[b] = lens[b] + block_len
+        for p in range(block_len):
+            t = int(lens[b]) + p
+            pos[b, p] = t
+            pg = t // page
+            if pg < bt.shape[1] and bt[b, pg] >= 0:
+                slots[b, p] = bt[b, pg] * page + t % page
+    return pos, slots, ctx
+
+
+def masked_rows(tokens, phase, mask_token_id: int, cap: int):
+    """Flat indices of the still-masked positions of the denoising lanes, in order, padded to `cap`
+    with the first entry (0 when there is none); and their count."""
+    tokens, phase = np.asarray(tokens), np.asarray(phase)
+    found = [b * tokens.shape[1] + p for b in range(tokens.shape[0]) if phase[b] == DENOISING
+             for p in range(tokens.shape[1]) if tokens[b, p] == mask_token_id]
+    fill = found[0] if found else 0
+    rows = (found + [fill] * cap)[:cap]
+    return np.asarray(rows, dtype=np.int64), len(found)
+
+
+def block_advance(tokens, transfer, step_map, step, phase, lens, first_len, max_new, stop_ids, mask_token_id: int):
+    """What follows the selection, per lane: Sampler.forward's bookkeeping (layers/sampler.py:56-59) and
+    Scheduler.postprocess (engine/scheduler.py:65-82).  Works on copies; returns the new
+    (tokens, step_map, step, phase, lens), the appended (tokens, steps) per lane (None when nothing
+    was appended) and the status rows (phase, len, masked left, committed in this pass)."""
+    tokens, step_map = np.array(tokens), np.array(step_map)
+    step, phase, lens = np.array(step), np.array(phase), np.array(lens)
+    transfer = np.asarray(transfer, dtype=bool)
+    appended, status = [], []
+    S = tokens.shape[1]
+    for b in range(tokens.shape[0]):
+        if phase[b] == IDLE:
+            appended.append(None)
+            status.append((IDLE, None, 0, 0))
+            continue
+        step_map[b][transfer[b]] = step[b]
+        step[b] += 1
+        moved = int(transfer[b].sum())
+        if phase[b] == DENOISING:
+            left = int((tokens[b] == mask_token_id).sum())
+            if left == 0:
+                phase[b] = CACHING
+            appended.append(None)
+        else:
+            stop = any(s >= 0 and (tokens[b] == s).any() for s in stop_ids[b])
+            appended.append((tokens[b].copy(), step_map[b].copy()))
+            tokens[b] = mask_token_id
+            lens[b] += S
+            left = S
+            phase[b] = IDLE if (stop or lens[b] - first_len[b] >= max_new[b]) else DENOISING
+        status.append((int(phase[b]), int(lens[b]), 0 if phase[b] == IDLE else left, moved))
+    return tokens, step_map, step, phase, lens, appended, status

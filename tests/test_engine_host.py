@@ -148,3 +148,82 @@ def test_preemption_when_the_page_pool_runs_out():
         assert s.status == SequenceStatus.FINISHED and s.num_completion_tokens == 288
         assert s.completion_token_ids == [10 + p for p in range(32)] * 9
     assert len(eng.block_manager.free) == 4 and not eng.running and not eng.waiting
+
+
+# ---- the per-lane block state machine of the device loop, on the CPU ---------------------------------------
+def test_oracle_block_prepare_is_get_slots_per_lane():
+    lens, phase = [250, 10, 700, 0], [1, 2, 0, 1]
+    bt = np.array([[7, 2, -1, -1], [5, -1, -1, -1], [1, 3, 4, -1], [6, -1, -1, -1]], dtype=np.int32)
+    pos, slots, ctx = oracle.block_prepare(lens, phase, bt, PAGE, 32)
+    assert ctx.tolist() == [282, 42, 0, 32]
+    for b in (0, 1, 3):
+        assert pos[b].tolist() == list(range(lens[b], lens[b] + 32))
+        assert slots[b].tolist() == oracle.get_slots([int(x) for x in bt[b] if x >= 0], lens[b], lens[b] + 32)
+    assert (slots[2] == -1).all() and (pos[2] == 0).all()                  # idle lane = graph padding
+    # a block that runs past the last page of the table has no slot there
+    _, s2, _ = oracle.block_prepare([250], [1], np.array([[9, -1]], dtype=np.int32), PAGE, 32)
+    assert s2[0, :6].tolist() == [9 * PAGE + 250 + i for i in range(6)] and (s2[0, 6:] == -1).all()
+
+
+def test_oracle_masked_rows():
+    tok = np.full((3, 8), 5)
+    tok[0, [1, 6]] = MASK
+    tok[1, :] = MASK                                                       # idle lane: not listed
+    tok[2, 3] = MASK
+    rows, n = oracle.masked_rows(tok, [1, 0, 1], MASK, 6)
+    assert n == 3 and rows.tolist() == [1, 6, 19, 1, 1, 1]
+    rows, n = oracle.masked_rows(tok, [2, 0, 2], MASK, 4)                  # caching lanes have nothing masked to project
+    assert n == 0 and rows.tolist() == [0, 0, 0, 0]
+    rows, n = oracle.masked_rows(tok, [1, 1, 1], MASK, 2)                  # more than the list holds: count says so
+    assert n == 11 and rows.tolist() == [1, 6]
+
+
+@pytest.mark.parametrize("k,peak", [(1, 0.0), (4, 0.0), (8, 0.0), (4, 30.0)])
+def test_oracle_block_advance_runs_the_same_generation_as_the_host_engine(k, peak):
+    """select_transfer + block_advance, pass after pass, against the host engine's Sequence / postprocess on the
+    same scripted confidences: same pass count (the closed form), same tokens, same step maps."""
+    model = ScriptedModel(peak=peak)
+    eng = _engine(model)
+    budgets = [64, 96]
+    sp = [SamplingParams(max_new_tokens=b, ignore_eos=True, transfer_count=k) for b in budgets]
+    seqs = [eng.add_request(list(range(300)), sp[0]), eng.add_request(list(range(40)), sp[1])]
+    eng.generate()
+
+    S = 32
+    logits = model.compute_logits(torch.zeros(2, S, 8)).double().numpy()      # the scripted logits of a decode pass
+    _, conf = oracle.confidence_argmax(logits)
+    x0 = logits.argmax(-1)
+    tokens = np.full((2, S), MASK, dtype=np.int64)
+    step_map = np.zeros((2, S), dtype=np.int32)
+    step, phase, lens = np.zeros(2, dtype=np.int32), np.array([1, 1]), np.array([300, 40])
+    first, stop = np.array([300, 40]), np.full((2, 4), -1)
+    out_tok, out_step, passes = [[], []], [[], []], 0
+    while (phase != 0).any():
+        transfer = oracle.select_transfer(conf.astype(np.float32), (tokens == MASK) & (phase[:, None] == 1), 0.9, k)
+        tokens = np.where(transfer, x0, tokens)
+        tokens, step_map, step, phase, lens, appended, status = oracle.block_advance(
+            tokens, transfer, step_map, step, phase, lens, first, np.array(budgets), stop, MASK)
+        for b, a in enumerate(appended):
+            if a is not None:
+                out_tok[b] += a[0].tolist()
+                out_step[b] += a[1].tolist()
+        passes += 1
+    per_block = 2 if peak else oracle.expected_passes(S, k, 1)
+    assert passes == 3 * per_block                                           # the longer request: three blocks
+    assert passes == len(model.calls)                                        # the host engine's prefill pass is its first denoising pass
+    for b, s in enumerate(seqs):
+        assert out_tok[b] == s.completion_token_ids and out_step[b] == s.step_map
+        assert lens[b] == s.num_tokens
+
+
+def test_oracle_block_advance_stop_token_and_idle_lanes():
+    S = 32
+    tokens = np.tile(np.arange(10, 10 + S), (3, 1)).astype(np.int64)          # complete blocks
+    zeros = np.zeros((3, S), dtype=bool)
+    stop = np.array([[17, -1, -1, -1], [-1, -1, -1, -1], [17, -1, -1, -1]])
+    t, m, step, phase, lens, appended, status = oracle.block_advance(
+        tokens, zeros, np.zeros((3, S), dtype=np.int32), [4, 4, 4], [2, 2, 0], [5, 5, 5], [5, 5, 5], [320, 320, 320], stop, MASK)
+    assert phase.tolist() == [0, 1, 0] and lens.tolist() == [37, 37, 5]      # lane 0 stops, lane 1 goes on, lane 2 was idle
+    assert appended[2] is None and appended[0][0].tolist() == list(range(10, 42))
+    assert (t[0] == MASK).all() and (t[2] == tokens[2]).all() and step.tolist() == [5, 5, 4]
+    assert status[1] == (1, 37, S, 0)

@@ -354,3 +354,34 @@ def test_prefill_sequence_bounds_are_clipped_to_the_tensors(dev):
     torch.cuda.synchronize()
     ref = oracle.staircase_attn_varlen(q[:120], k[:120], v[:120], torch.tensor([0, 120], dtype=torch.int32), 32)
     assert (o[:60].float().cpu() - ref[:60]).abs().max().item() < TOL
+
+
+@pytest.mark.parametrize("ctxs", [[700, 300], [3000, 2500, 40]])
+def test_paged_sequence_without_a_valid_page_yields_zeros(dev, ctxs):
+    """A sequence whose page ids are all invalid (-1 or past the pool) has no key to attend to: its
+    rows are zeros, like a sequence of context 0, whether it is split or not; the others are untouched."""
+    import mdx
+    g = torch.Generator().manual_seed(91)
+    q, kc, vc, bt, lens = _paged_inputs(g, ctxs)
+    bad = bt.clone()
+    bad[0] = -1
+    bad[0, 0] = kc.shape[0] + 5
+    scale = 1 / math.sqrt(q.shape[-1])
+    for counters in (None, False):
+        o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens.to(dev), block_table=bad.to(dev),
+                                        softmax_scale=scale, causal=False, counters=counters).float().cpu()
+        assert o[0].abs().max().item() == 0 and not torch.isnan(o).any()
+        ref = oracle.paged_block_attn(q[1:], kc, vc, bt[1:], lens[1:], scale)
+        assert (o[1:] - ref).abs().max().item() < 2e-2
+
+
+def test_prefill_default_grid_bound_covers_every_row(dev):
+    """max_seqlen only sizes the grid: leaving it out (the bound is then the total token count) and giving
+    the exact maximum produce the same output, bit for bit, on every row."""
+    import mdx
+    g = torch.Generator().manual_seed(92)
+    lens = [900, 40, 333]
+    q, k, v, cu = _packed(g, lens, 16, 8)
+    a = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    b = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, max_seqlen=max(lens))
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))

@@ -84,10 +84,12 @@ def test_engine_is_deterministic_and_independent_of_page_placement(dev):
     assert outs[0] == outs[1]
 
 
-def test_decode_graph_replays_match_eager(dev):
-    """A captured decode forward, replayed several times on different blocks, lengths and page
-    tables with eager work and synchronisations in between, equals the eager forward bit for bit."""
-    from mdx.context import set_context
+def test_device_loop_forward_replays_match_eager(dev):
+    """The captured forward of the device loop (pass inputs computed on the device from lengths and page tables,
+    then the decoder), replayed on different blocks, lengths and page tables with eager work and
+    synchronisations in between: its pass inputs equal the host's prepare_decode and its hidden states equal
+    the eager forward on the same inputs, bit for bit."""
+    from mdx.context import reset_context, set_context
     from mdx.engine import BlockDiffusionEngine, SamplingParams
     cfg, model = _tiny(dev)
     eng = BlockDiffusionEngine(model, num_pages=24, shuffle_pages_seed=7, decode_graphs=True, max_model_len=1024)
@@ -100,22 +102,57 @@ def test_decode_graph_replays_match_eager(dev):
             blk = torch.full((32,), cfg.mask_token_id, dtype=torch.int64)
             blk[: 4 * rep] = torch.randint(0, 900, (4 * rep,), generator=g)
             s.current_denoising_block = blk
-        hidden = eng._run_decode_graph(seqs)[0].clone()
+            eng.block_manager.may_append(s)
+        gr = eng._load_lanes(seqs)                         # three sequences run in the lanes captured for four
+        assert gr["bs"] == 4
+        gr["fwd"].replay()
+        hidden = gr["hidden"].clone()
         torch.cuda.synchronize()
-        ids, pos = eng.prepare_decode(seqs)                # eager, its own tensors for the three sequences
-        gr = eng._graphs[4]                                # three sequences run in the graph captured for four
+        ids, pos = eng.prepare_decode(seqs)                # the host's version of the same pass inputs
+        from mdx.context import get_context
+        ctx = get_context()
         assert torch.equal(gr["ids"][:3], ids) and torch.equal(gr["pos"][:3], pos)
-        assert gr["lens"][3].item() == 0 and (gr["slots"][3] == -1).all()      # the padding row
-        set_context(False, slot_mapping=gr["slots"], context_lens=gr["lens"], block_tables=gr["bt"], block_size=32)
+        assert torch.equal(gr["slots"][:3], ctx.slot_mapping) and torch.equal(gr["ctx"][:3], ctx.context_lens)
+        assert gr["ctx"][3].item() == 0 and (gr["slots"][3] == -1).all()        # the idle lane
+        set_context(False, slot_mapping=gr["slots"], context_lens=gr["ctx"], block_tables=gr["bt"], block_size=32)
         ref = model(model.embed(gr["ids"].clone()), gr["pos"].clone())          # same launch geometry as the capture
+        reset_context()
         torch.cuda.synchronize()
         assert torch.equal(hidden, ref), f"replay {rep}: max diff {(hidden.float() - ref.float()).abs().max().item()}"
-        assert hidden[3].abs().sum().item() == hidden[3].abs().sum().item()     # padding row: finite
+        assert torch.isfinite(hidden[3].float()).all()                          # idle lane: finite
+        eng._loaded = None
         if rep == 2:                                       # sequences grow between replays
             for s in seqs:
                 s.current_denoising_block = torch.randint(0, 900, (32,), generator=g)
                 s.append_block()
                 eng.block_manager.may_append(s)
+
+
+def test_device_loop_generates_like_the_host_driven_engine(dev):
+    """The same requests through the host-driven engine and through the device loop, with and without the one-pass
+    lag of the status reads and with the projection on all rows or on the masked rows: same number of passes, and
+    the same tokens and step maps up to near-ties (the lanes' page tables have their full width, which moves the
+    split points of the paged attention)."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for kw in (dict(decode_graphs=False), dict(decode_graphs=True, replay_ahead=False), dict(decode_graphs=True),
+               dict(decode_graphs=True, masked_rows_only=False)):
+        eng = BlockDiffusionEngine(model, num_pages=24, shuffle_pages_seed=9, max_model_len=1024, **kw)
+        g = torch.Generator().manual_seed(12)
+        seqs = [eng.add_request(torch.randint(0, 900, (n,), generator=g).tolist(),
+                                SamplingParams(max_new_tokens=96, ignore_eos=True, transfer_count=4, temperature=t))
+                for n, t in ((250, 1.0), (33, 0.8), (140, 1.2))]
+        eng.generate()
+        assert all(s.num_completion_tokens == 96 and len(s.step_map) == 96 for s in seqs)
+        assert eng.stats["decode_passes"] == 3 * 9 - 1 and eng.stats["committed_tokens"] == 3 * 96
+        assert len(eng.block_manager.free) == 24 and not eng.running
+        outs.append([(s.completion_token_ids, list(s.step_map)) for s in seqs])
+    for other in outs[1:]:
+        for (ta, ma), (tb, mb) in zip(outs[0], other):
+            assert sum(int(a == b) for a, b in zip(ta, tb)) >= 90
+            assert sum(int(a == b) for a, b in zip(ma, mb)) >= 90
+    assert outs[1] == outs[2]                               # the lag is pure scheduling
 
 
 def test_engine_with_decode_graphs_generates_like_eager(dev):

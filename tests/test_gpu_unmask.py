@@ -196,3 +196,24 @@ def test_confidence_extreme_logits(dev):
     # to a percent, while the kernel scales the exact difference to the maximum: the argmax must
     # still agree exactly, the probability within that rounding.
     _check_conf(dev, logits.bfloat16(), temps=torch.tensor([0.05, 1.0, 7.0]), rtol=3e-2)
+
+
+def test_rows_without_a_finite_logit_are_never_committed(dev):
+    """A row of -inf logits has no softmax: token 0 with confidence 0, with and without noise and
+    through the split-row path, so neither selection rule can pick it over a real candidate."""
+    import mdx
+    g = torch.Generator().manual_seed(17)
+    logits = (torch.randn(1, 4, 151936, generator=g) * 3).bfloat16()
+    logits[0, 1] = float("-inf")
+    logits[0, 3, 5:] = float("-inf")                      # a row with a few finite entries is an ordinary row
+    x0, p = mdx.confidence_argmax(logits.to(dev))
+    ex0, ep = oracle.confidence_argmax(_f64(logits[:, [0, 2, 3]]))
+    assert np.array_equal(x0.cpu().numpy()[:, [0, 2, 3]], ex0)
+    np.testing.assert_allclose(p.cpu().numpy()[:, [0, 2, 3]], ep, rtol=2e-5)
+    assert x0[0, 1].item() == 0 and p[0, 1].item() == 0.0
+    noise = torch.zeros(1, 4, 151936)
+    x0n, pn = mdx.confidence_argmax(logits.to(dev), None, noise.to(dev))
+    assert x0n[0, 1].item() == 0 and pn[0, 1].item() == 0.0
+    tokens = torch.full((1, 4), MASK_ID, dtype=torch.int64, device=dev)
+    _, _, transfer, count = mdx.unmask_step(logits.to(dev), tokens, MASK_ID, 0.9, 3)
+    assert transfer.cpu().tolist() == [[True, False, True, True]] and int(count[0]) == 3
