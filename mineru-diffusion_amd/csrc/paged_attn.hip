@@ -41,6 +41,21 @@ __device__ __forceinline__ int wave_sum(int x) {
     return __builtin_amdgcn_readfirstlane(x);      // the same in every lane: say so to the compiler
 }
 
+// Partials that another workgroup of the same launch reads (single-launch merge) travel with
+// agent-scope accesses: such a store is written through to memory and such a load does not take a line
+// that this XCD's L2 may still hold from an earlier launch.  That makes them visible across the XCDs'
+// L2 caches without the release fence (a write-back walk of the whole L2) that ordinary stores would need.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+__device__ __forceinline__ void store_agent(float* p, f32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ f32x4 load_agent(const float* p) {
+    f32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void wait_vector_memory() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 struct PagedParams {
     const __bf16* q; __bf16* o; const __bf16* k_cache; const __bf16* v_cache;
     int64_t q_sb, q_ss, q_sh, o_sb, o_ss, o_sh;     // element strides
@@ -66,6 +81,7 @@ struct PagedParams {
 
 // Merges the nv split partials of query s of (sequence b, head hq); the caller's 8 threads c = 0..7
 // of a query take 16 consecutive d values each.
+template <bool AGENT>
 __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, int nv)
 {
     const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
@@ -75,15 +91,31 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
     for (int e = 0; e < 16; ++e) acc[e] = 0.f;
     for (int i0 = 0; i0 < nv; i0 += 4) {
         float m[4], l[4];
-        float4 po[4][4];
+        f32x4 po[4][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int64_t slot = slot0 + min(i0 + i, nv - 1);
-            m[i] = P.part_ml[(slot * 2 + 0) * kMaxSq + s];
-            l[i] = P.part_ml[(slot * 2 + 1) * kMaxSq + s];
-            const float4* src = reinterpret_cast<const float4*>(P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16);
+            const float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + s;
+            const float* src = P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16;
+            if (AGENT) {
+                m[i] = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                l[i] = __hip_atomic_load(ml + kMaxSq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) po[i][k] = src[k];
+                for (int k = 0; k < 4; ++k) po[i][k] = load_agent(src + 4 * k);
+            } else {
+                m[i] = ml[0];
+                l[i] = ml[kMaxSq];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) po[i][k] = *reinterpret_cast<const f32x4*>(src + 4 * k);
+            }
+        }
+        if (AGENT) {
+            // the asm loads are invisible to the compiler's own counting: wait here, and tie every loaded
+            // value to the wait so that no use of it can be scheduled above it
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(po[i][k]) :: "memory");
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
@@ -351,33 +383,40 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float4 out = make_float4(st.o[0][dt][4 * g], st.o[0][dt][4 * g + 1], st.o[0][dt][4 * g + 2], st.o[0][dt][4 * g + 3]);
-                *reinterpret_cast<float4*>(po + d_of_reg(dt, 4 * g, H)) = out;
+                const f32x4 out = {st.o[0][dt][4 * g], st.o[0][dt][4 * g + 1], st.o[0][dt][4 * g + 2], st.o[0][dt][4 * g + 3]};
+                if (P.arrive) store_agent(po + d_of_reg(dt, 4 * g, H), out);
+                else *reinterpret_cast<f32x4*>(po + d_of_reg(dt, 4 * g, H)) = out;
             }
         if (H == 0) {
-            P.part_ml[(slot * 2 + 0) * kMaxSq + r] = st.m[0];
-            P.part_ml[(slot * 2 + 1) * kMaxSq + r] = st.l[0];
+            float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + r;
+            if (P.arrive) {
+                __hip_atomic_store(ml, st.m[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(ml + kMaxSq, st.l[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                ml[0] = st.m[0];
+                ml[kMaxSq] = st.l[0];
+            }
         }
     }
     if (!P.arrive) return;                       // two-launch mode: the combine kernel follows
 
     // ---- single-launch mode: the last split of this (sequence, head group) to arrive merges them ----
-    // Release: every writer makes its partials visible device-wide before the workgroup counts
-    // itself in; acquire: the workgroup that finds itself last drops stale cache lines before it
-    // reads the others' partials.  Nobody waits for anybody: a workgroup that is not last leaves.
+    // Every writer waits until its (written-through) partials have reached memory, then the workgroup
+    // counts itself in; the workgroup that finds itself last reads all partials of the pair with
+    // agent-scope loads.  No cache-wide fence on either side, and nobody waits for anybody: a
+    // workgroup that is not last leaves.
     __shared__ int i_am_last;
-    __threadfence();
+    wait_vector_memory();
     __syncthreads();
     float* counter = P.arrive + (int64_t)b * gridDim.x + hg;
     if (tid == 0) i_am_last = atomicAdd(counter, 1.0f) == (float)(n_valid_splits - 1) ? 1 : 0;
     __syncthreads();
     if (!i_am_last) return;
-    __threadfence();
     for (int e = tid; e < HPW * 256; e += kThreads) {
         const int s = (e & 255) >> 3;
-        if (s < P.sq) combine_query(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
+        if (s < P.sq) combine_query<true>(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
     }
-    if (tid == 0) *counter = 0.f;                // ready for the next launch
+    if (tid == 0) __hip_atomic_store(counter, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
 
 // One workgroup per (sequence, head): merges the split partials of its 32 queries; thread t takes
@@ -394,7 +433,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     if (nv <= 1) return;                                   // written directly by the attention kernel
     const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
     if (s >= P.sq) return;
-    combine_query(P, b, hq, s, c, nv);
+    combine_query<false>(P, b, hq, s, c, nv);
 }
 
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
@@ -504,11 +543,14 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
         P.part_o = static_cast<float*>(workspace);
         P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
         if (device_span) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
-        // Counting in costs every split workgroup a device-wide release (a walk of its XCD's L2 for dirty
-        // lines), which a launch of hundreds of split workgroups pays a hundred times over (config 2:
-        // 48 -> 145 us), while a launch whose sequences stay whole pays nothing and saves the combine
-        // launch (batch 32: 62 -> 60 us).  So only the launches that cut nothing but outliers
-        // (device_span) take the single-launch path; the others keep the combine kernel.
+        // Single launch: the partials are written through with agent-scope stores and read back with
+        // agent-scope loads, so counting in costs a workgroup the wait for its own stores and one atomic,
+        // not a device-wide release (a write-back walk of its XCD's L2).  Where only outliers are cut
+        // (device_span) that beats the combine launch (ragged batch of 32: 93 -> 80 us, and a launch
+        // whose sequences stay whole pays nothing).  Where every sequence is split the merges all fall
+        // at the end of the launch, one after the other behind the written-through stores (config 2:
+        // 61 us against 49 with the combine launch; with full release fences it was 145), so those
+        // launches keep the combine kernel.
         if (single_launch && device_span) {
             const int64_t need_c = (int64_t)bs * (num_q_heads / HPW) * (int64_t)sizeof(float);
             MDX_REQUIRE(counters && counter_bytes >= need_c, MDX_EWORKSPACE,
