@@ -33,7 +33,7 @@ extern "C" {
 #define MDX_ELAUNCH      -4        /* the HIP runtime refused the launch */
 
 #define MDX_BF16 0                 /* q/k/v/o, the caches, the layer ops, the logits */
-#define MDX_F16  1                 /* logits only */
+#define MDX_F16  1                 /* q/k/v/o and the caches of the two attention calls, the logits */
 #define MDX_F32  2                 /* logits only */
 
 typedef void* mdx_stream_t;        /* hipStream_t */
@@ -81,7 +81,8 @@ int mdx_store_kvcache(const void* key, const void* value,
  * (their o rows keep what they held; the lengths are on the device, so the
  * call cannot check this).  total_tokens is always a valid bound; the
  * reference interface has no such argument.  Supported: d == 128, dtype
- * MDX_BF16.
+ * MDX_BF16 or MDX_F16 (the reference kernel takes q's dtype, :179-197; fp16
+ * runs the one-head-per-wavefront kernel, about 0.8 x the bf16 rate).
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                               int64_t q_stride_t, int64_t q_stride_h,
@@ -114,7 +115,7 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * kernel picks it from the lengths); its size comes from
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
  * contents need no initialisation.
- * Supported: d == 128, Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0, MDX_BF16.
+ * Supported: d == 128, Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0, MDX_BF16 or MDX_F16.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
                                              int32_t num_kv_heads, int32_t head_dim,

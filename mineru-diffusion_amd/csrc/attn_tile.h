@@ -1,5 +1,6 @@
 // Wavefront-level building block shared by the two attention kernels
-// (staircase block-prefill and paged single-block decode), head_dim 128, bf16.
+// (staircase block-prefill and paged single-block decode), head_dim 128, bf16 or fp16 (pointers are
+// typed __bf16 throughout as "16-bit element"; the element type E of a kernel says what the bits mean).
 //
 // One wavefront owns 32 query rows (one MFMA column tile) of NH query heads that share a KV
 // head and walks over keys 32 at a time:
@@ -32,6 +33,7 @@
 namespace mdx_attn {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -42,6 +44,21 @@ constexpr int kLdsPitch = kRowBytes + 16;    // 272: consecutive rows shift by 4
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kMinusBig = -1.0e30f;        // finite initial running max (avoids inf - inf)
 constexpr float kMaxSlack = 8.0f;            // running max may lag by up to 2^8 before O is rescaled
+
+// The two 16-bit element types the tile code runs in.  Everything that moves K/V/Q bytes is type-blind
+// (16-byte copies); the type decides the MFMA instruction and the two float -> element conversions
+// (probabilities, output).
+template <typename E> struct Elem16;
+template <> struct Elem16<__bf16> {
+    typedef bf16x8 vec8;
+    typedef __attribute__((ext_vector_type(4))) __bf16 vec4;
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Elem16<_Float16> {
+    typedef f16x8 vec8;
+    typedef __attribute__((ext_vector_type(4))) _Float16 vec4;
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
 
 __device__ __forceinline__ int key_of_reg(int i, int H) {
     return 16 * (i >> 3) + 4 * (i & 3) + 2 * H + ((i >> 2) & 1);
@@ -93,9 +110,10 @@ struct WaveState {
 // n0 .. n0+NSUB*32-1 of tiles with row pitch kLdsPitch.
 
 // S^T = K Q^T.  q[h][ks] are the B-operand fragments of Q^T for d = 16ks .. 16ks+15.
-template <int NH, int NSUB>
-__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8 (&q)[NH][8], f32x16 (&s)[NH][NSUB], int lane)
+template <typename E, int NH, int NSUB>
+__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const typename Elem16<E>::vec8 (&q)[NH][8], f32x16 (&s)[NH][NSUB], int lane)
 {
+    typedef typename Elem16<E>::vec8 vec8;
     const int H = lane >> 5, r = lane & 31;
 #pragma unroll
     for (int h = 0; h < NH; ++h)
@@ -108,10 +126,10 @@ __device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8
     for (int ks = 0; ks < 8; ++ks) {
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kbase + u * 32 * kLdsPitch + ks * 32);
+            const vec8 kf = *reinterpret_cast<const vec8*>(kbase + u * 32 * kLdsPitch + ks * 32);
 #pragma unroll
             for (int h = 0; h < NH; ++h)
-                s[h][u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q[h][ks], s[h][u], 0, 0, 0);
+                s[h][u] = Elem16<E>::mfma(kf, q[h][ks], s[h][u]);
         }
     }
 }
@@ -121,8 +139,8 @@ __device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const bf16x8
 // absolute index of LDS row n0; key_hi may differ per lane (per query), key_lo is uniform.
 // Produces the bf16 B-operand fragments p[h][u][t] of P^T and updates m, l and (when the
 // running max moves) rescales O.
-template <int NH, int NSUB, bool MASK>
-__device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], bf16x8 (&p)[NH][NSUB][2], WaveState<NH>& st, float c,
+template <typename E, int NH, int NSUB, bool MASK>
+__device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], typename Elem16<E>::vec8 (&p)[NH][NSUB][2], WaveState<NH>& st, float c,
                                               int lane, int key_abs0, int key_lo, int key_hi)
 {
     const int H = lane >> 5;
@@ -159,7 +177,7 @@ __device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], bf16x8 (&p)
                 for (int j = 0; j < 8; ++j) {
                     const float e = __builtin_amdgcn_exp2f(fmaf(s[h][u][8 * t + j], c, -m_new));
                     sum += e;
-                    p[h][u][t][j] = (__bf16)e;
+                    p[h][u][t][j] = (E)e;
                 }
         if (moved) {
             const float alpha = __builtin_amdgcn_exp2f(st.m[h] - m_new);
@@ -176,9 +194,10 @@ __device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], bf16x8 (&p)
 
 // O^T += V^T P^T.  The lane supplies the row address for the transposing read:
 // row 4*(i'/4) + 2H (+q), d chunk i'%4, with i' = lane % 16.
-template <int NH, int NSUB>
-__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const bf16x8 (&p)[NH][NSUB][2], WaveState<NH>& st, int lane)
+template <typename E, int NH, int NSUB>
+__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const typename Elem16<E>::vec8 (&p)[NH][NSUB][2], WaveState<NH>& st, int lane)
 {
+    typedef typename Elem16<E>::vec8 vec8;
     const int H = lane >> 5, ip = lane & 15, gi = (lane >> 4) & 1;
     const lds_char* vbase = (const lds_char*)lds_v + (n0 + 4 * (ip >> 2) + 2 * H) * kLdsPitch + (gi * 16 + (ip & 3) * 4) * 2;
 #pragma unroll
@@ -191,23 +210,23 @@ __device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const bf16x8
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a);
                 const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + kLdsPitch));
                 const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                const bf16x8 vf = __builtin_bit_cast(bf16x8, both);
+                const vec8 vf = __builtin_bit_cast(vec8, both);
 #pragma unroll
                 for (int h = 0; h < NH; ++h)
-                    st.o[h][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, p[h][u][t], st.o[h][dt], 0, 0, 0);
+                    st.o[h][dt] = Elem16<E>::mfma(vf, p[h][u][t], st.o[h][dt]);
             }
 }
 
 // All three phases back to back.
-template <int NH, int NSUB, bool MASK>
-__device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, int n0, const bf16x8 (&q)[NH][8],
+template <typename E, int NH, int NSUB, bool MASK>
+__device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, int n0, const typename Elem16<E>::vec8 (&q)[NH][8],
                                           WaveState<NH>& st, float c, int lane, int key_abs0, int key_lo, int key_hi)
 {
     f32x16 s[NH][NSUB];
-    bf16x8 p[NH][NSUB][2];
-    qk_phase<NH, NSUB>(lds_k, n0, q, s, lane);
-    softmax_phase<NH, NSUB, MASK>(s, p, st, c, lane, key_abs0, key_lo, key_hi);
-    pv_phase<NH, NSUB>(lds_v, n0, p, st, lane);
+    typename Elem16<E>::vec8 p[NH][NSUB][2];
+    qk_phase<E, NH, NSUB>(lds_k, n0, q, s, lane);
+    softmax_phase<E, NH, NSUB, MASK>(s, p, st, c, lane, key_abs0, key_lo, key_hi);
+    pv_phase<E, NH, NSUB>(lds_v, n0, p, st, lane);
 }
 
 // d index held by accumulator register i of O^T tile dt in half-wave H.
@@ -215,14 +234,15 @@ __device__ __forceinline__ int d_of_reg(int dt, int i, int H) { return dt * 32 +
 
 // Loads the Q^T B-operand fragments of one head for this lane's query row
 // (row pointer may be null: zeros).  q_row points at Q[query, head, 0].
-__device__ __forceinline__ void load_q(bf16x8 (&q)[8], const __bf16* q_row, int H) {
+template <typename V8>
+__device__ __forceinline__ void load_q(V8 (&q)[8], const __bf16* q_row, int H) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
         if (q_row) {
-            q[ks] = *reinterpret_cast<const bf16x8*>(q_row + ks * 16 + H * 8);
+            q[ks] = *reinterpret_cast<const V8*>(q_row + ks * 16 + H * 8);
         } else {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[ks][j] = (__bf16)0.f;
+            for (int j = 0; j < 8; ++j) q[ks][j] = 0;
         }
     }
 }

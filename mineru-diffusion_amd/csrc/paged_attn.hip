@@ -81,7 +81,7 @@ struct PagedParams {
 
 // Merges the nv split partials of query s of (sequence b, head hq); the caller's 8 threads c = 0..7
 // of a query take 16 consecutive d values each.
-template <bool AGENT>
+template <typename E, bool AGENT>
 __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, int nv)
 {
     const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
@@ -140,21 +140,21 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
         }
     }
     const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;   // no valid key at all (every page id invalid): zeros, like a context of 0
-    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+    typedef typename Elem16<E>::vec8 vec8;
     __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        bf16x8_t out;
+        vec8 out;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) out[e] = (__bf16)(acc[8 * h + e] * inv);
-        *reinterpret_cast<bf16x8_t*>(dst + 8 * h) = out;
+        for (int e = 0; e < 8; ++e) out[e] = (E)(acc[8 * h + e] * inv);
+        *reinterpret_cast<vec8*>(dst + 8 * h) = out;
     }
 }
 
 // WAVES = 4 (two workgroups per CU) or 8 (one workgroup per CU, 128-key tiles: for launches with about
 // one workgroup per CU, where a CU would otherwise hold four wavefronts only).  Tiles hold 32 keys per
 // key slice (WAVES / HPW slices); two 64-key tile buffers fit a CU twice, two 128-key ones once.
-template <int HPW, int DEPTH, int WAVES>
+template <typename E, int HPW, int DEPTH, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_block_attn_kernel(const PagedParams P)
 {
     constexpr int kThreads = 64 * WAVES;
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     const int kvh = (hg * HPW) / P.heads_per_kv;
 
     const bool row_ok = r < P.sq;
-    bf16x8 q[1][8];
+    typename Elem16<E>::vec8 q[1][8];
     load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H);
 
     WaveState<1> st;
@@ -284,9 +284,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         // keys of an invalid page are excluded (not merely zeroed): the owning wavefront skips them
         if ((tile_pass_ok[t & 1] >> (kPassesPerSlice * kw)) & 1u) {
             if (key0 + 32 <= key_end)
-                attn_step<1, 1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<E, 1, 1, false>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
             else
-                attn_step<1, 1, true>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
+                attn_step<E, 1, 1, true>(lk, lk + kTileBytes, kw * 32, q, st, P.c, lane, key0, 0, key_end);
         }
     };
 
@@ -368,11 +368,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-                bf16x4 out;
+                typename Elem16<E>::vec4 out;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
-                *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+                for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
+                *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
             }
         return;
     }
@@ -414,7 +413,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     if (!i_am_last) return;
     for (int e = tid; e < HPW * 256; e += kThreads) {
         const int s = (e & 255) >> 3;
-        if (s < P.sq) combine_query<true>(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
+        if (s < P.sq) combine_query<E, true>(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
     }
     if (tid == 0) __hip_atomic_store(counter, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
@@ -424,6 +423,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
 // there are only bs * Hq workgroups to launch, which is what the common case costs when the
 // attention kernel decided that nothing had to be cut.  The kernel is a chain of memory latencies
 // (length -> partials -> output), not of bytes: the loads of four splits are issued together.
+template <typename E>
 __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
     const int hq = blockIdx.x % P.num_q_heads, b = blockIdx.x / P.num_q_heads;
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
     if (nv <= 1) return;                                   // written directly by the attention kernel
     const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
     if (s >= P.sq) return;
-    combine_query<false>(P, b, hq, s, c, nv);
+    combine_query<E, false>(P, b, hq, s, c, nv);
 }
 
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
@@ -499,7 +499,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && sq >= 0 && max_pages >= 0 && num_pages >= 0, MDX_EINVAL, "paged_block_attn: negative size");
-    MDX_REQUIRE(dtype == MDX_BF16, MDX_EUNSUPPORTED, "paged_block_attn: dtype %d (only bf16)", dtype);
+    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "paged_block_attn: dtype %d (bf16 or fp16)", dtype);
     MDX_REQUIRE(head_dim == kHeadDim, MDX_EUNSUPPORTED, "paged_block_attn: head_dim %d (only 128)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "paged_block_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
@@ -569,12 +569,21 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     // CU that holds a single workgroup still has two wavefronts per SIMD (batch 32 x 8 KV heads: 79 -> 69 us
     // on equal lengths); with more pairs than CUs the second round costs more than that gains.
     const bool eight = device_span && (int64_t)bs * (num_q_heads / HPW) <= 256;
-    if (HPW == 2 && eight) paged_block_attn_kernel<2, 2, 8><<<grid, 512, 0, stream>>>(P);
-    else if (HPW == 2)     paged_block_attn_kernel<2, 2, 4><<<grid, 256, 0, stream>>>(P);
-    else                   paged_block_attn_kernel<1, 1, 4><<<grid, 256, 0, stream>>>(P);
+    const unsigned n_combine = (unsigned)(bs * num_q_heads);
+    const bool two_launches = P.nsplit > 1 && !P.arrive;
+    if (dtype == MDX_F16) {
+        if (HPW == 2 && eight) paged_block_attn_kernel<_Float16, 2, 2, 8><<<grid, 512, 0, stream>>>(P);
+        else if (HPW == 2)     paged_block_attn_kernel<_Float16, 2, 2, 4><<<grid, 256, 0, stream>>>(P);
+        else                   paged_block_attn_kernel<_Float16, 1, 1, 4><<<grid, 256, 0, stream>>>(P);
+    } else {
+        if (HPW == 2 && eight) paged_block_attn_kernel<__bf16, 2, 2, 8><<<grid, 512, 0, stream>>>(P);
+        else if (HPW == 2)     paged_block_attn_kernel<__bf16, 2, 2, 4><<<grid, 256, 0, stream>>>(P);
+        else                   paged_block_attn_kernel<__bf16, 1, 1, 4><<<grid, 256, 0, stream>>>(P);
+    }
     int rc = mdx::check_launch("paged_block_attn");
-    if (rc != MDX_OK || P.nsplit == 1 || P.arrive) return rc;
-    paged_combine_kernel<<<(unsigned)(bs * num_q_heads), 256, 0, stream>>>(P);
+    if (rc != MDX_OK || !two_launches) return rc;
+    if (dtype == MDX_F16) paged_combine_kernel<_Float16><<<n_combine, 256, 0, stream>>>(P);
+    else                  paged_combine_kernel<__bf16><<<n_combine, 256, 0, stream>>>(P);
     return mdx::check_launch("paged_combine");
 }
 

@@ -101,6 +101,7 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
     return true;
 }
 
+template <typename E>
 __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const StaircaseParams P)
 {
     __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     const int ip = row_w0 + r;                                 // this lane's padded query row
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
-    bf16x8 q[1][8];
+    typename Elem16<E>::vec8 q[1][8];
     load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
 
     // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
@@ -183,11 +184,11 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         const int key0 = t * kTileKeys;
         if (key0 < wave_hi) {
             if (key0 >= pad && key0 + kTileKeys <= wave_hi_min) {
-                attn_step<1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else if (key0 + 32 < wave_hi) {
-                attn_step<1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             } else {
-                attn_step<1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
             }
         }
         if (t + 1 < n_tiles) {
@@ -206,11 +207,10 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-            bf16x4 out;
+            typename Elem16<E>::vec4 out;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) out[e] = (__bf16)(st.o[0][dt][4 * g + e] * inv);
-            *reinterpret_cast<bf16x4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+            for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
+            *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
         }
 }
 
@@ -329,7 +329,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(batch >= 0 && total_tokens >= 0 && max_seqlen >= 0, MDX_EINVAL, "staircase_attn: negative size");
-    MDX_REQUIRE(dtype == MDX_BF16, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (only bf16)", dtype);
+    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (bf16 or fp16)", dtype);
     MDX_REQUIRE(head_dim == kHeadDim, MDX_EUNSUPPORTED, "staircase_attn: head_dim %d (only 128)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "staircase_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
@@ -365,7 +365,8 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                                         : (int64_t)P.n_row_groups * batch;
     // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
     const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
-    const bool pairs = (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
+    // (the hand-scheduled pair kernel exists for bf16; fp16 runs the one-head kernel)
+    const bool pairs = dtype == MDX_BF16 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
@@ -374,8 +375,10 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
         MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
         staircase_pair_kernel<<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
+    } else if (dtype == MDX_F16) {
+        staircase_attn_kernel<_Float16><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     } else {
-        staircase_attn_kernel<<<(unsigned)grid, kThreads, 0, stream>>>(P);
+        staircase_attn_kernel<__bf16><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     }
     return mdx::check_launch("staircase_attn");
 }

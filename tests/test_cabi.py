@@ -63,7 +63,7 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     assert sa(d=64) == -2 and b"head_dim" in L.mdx_last_error()
     assert sa(S=48) == -1 and b"staircase_size" in L.mdx_last_error()
     assert sa(hq=12) == -1
-    assert sa(dtype=1) == -2
+    assert sa(dtype=2) == -2                                   # fp32 q/k/v: the attention runs on 16-bit elements only
     assert sa(scale=-1.0) == -1
     pa = lambda **kw: L.mdx_paged_block_attn(                                                  # noqa: E731
         one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,

@@ -385,3 +385,35 @@ def test_prefill_default_grid_bound_covers_every_row(dev):
     a = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
     b = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, max_seqlen=max(lens))
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+@pytest.mark.parametrize("hq,hkv", [(16, 8), (3, 1)])
+def test_fp16_prefill_and_decode(dev, hq, hkv):
+    """The reference kernel computes in q's dtype (block_prefill_attention_v2.py:179-197) and flash-attn takes fp16
+    as well: the same two calls on fp16 tensors, against the fp32 oracle on the same values (max-abs < 2e-2),
+    lengths that are no multiple of the block, a split and an unsplit paged sequence."""
+    import mdx
+    g = torch.Generator().manual_seed(160 + hq)
+    lens = [333, 64, 1000]
+    N = sum(lens)
+    q = torch.randn(N, hq, 128, generator=g).half()
+    k = torch.randn(N, hkv, 128, generator=g).half()
+    v = torch.randn(N, hkv, 128, generator=g).half()
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    assert o.dtype == torch.float16
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
+    # against the bf16 kernel on the same values rounded to bf16: two roundings apart at most
+    for ctxs in ([700, 4128, 33], [2300] * 4):
+        qd, kc, vc, bt, lens_d = _paged_inputs(g, ctxs, hq=hq, hkv=hkv)
+        qd, kc, vc = qd.half(), kc.half(), vc.half()
+        scale = 1 / math.sqrt(128)
+        od = mdx.flash_attn_with_kvcache(qd.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens_d.to(dev), block_table=bt.to(dev),
+                                         softmax_scale=scale, causal=False)
+        assert od.dtype == torch.float16
+        refd = oracle.paged_block_attn(qd, kc, vc, bt, lens_d, scale)
+        assert (od.float().cpu() - refd).abs().max().item() < TOL
+        od2 = mdx.flash_attn_with_kvcache(qd.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens_d.to(dev), block_table=bt.to(dev),
+                                          softmax_scale=scale, causal=False, counters=False)
+        assert torch.equal(od.view(torch.int16), od2.view(torch.int16))
