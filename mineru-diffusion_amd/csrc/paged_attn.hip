@@ -20,8 +20,12 @@
 //    HPW heads that share a KV head (2 for grouped-query attention) times
 //    KW = 4/HPW key slices of 32 keys.  Two workgroups share a CU.
 //  * K/V tiles of 32*KW keys travel global -> registers -> LDS with 16-byte
-//    coalesced loads; two tiles are in flight in registers while a third is
-//    consumed from the double-buffered LDS, so HBM latency stays covered.
+//    coalesced loads into two register sets while a third tile is consumed from
+//    the double-buffered LDS.  (As compiled, a stage waits for every load the
+//    wavefront has outstanding, because the fetch of the younger tile sits under
+//    a condition; making all fetches unconditional, so that the wait leaves the
+//    younger tile in flight, was measured and changes nothing: the depth of the
+//    load queue is not what bounds this kernel.)
 //  * the KW wavefront states of a head are merged through LDS, then either
 //    written as the final output (single split) or as an fp32 partial
 //    (m, l, O) that a second, small kernel combines.
@@ -241,10 +245,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     const int chunk = tid & 15, trow = tid >> 4;    // one pass stages kRowsPerPass rows
     const int n_tiles = (key_end - key_begin + kTileKeys - 1) / kTileKeys;
     // kRowsPerPass (16 or 32) consecutive keys starting at a multiple of that never straddle a page (page_size % 32 == 0):
-    // each pass looks its page up once.  The loads are unconditional (rows past the context or on
-    // an invalid page id read row `trow` of page 0 instead and are zeroed when they reach LDS), so
-    // the number of loads in flight is known exactly and waiting for one register set does not
-    // drain the other.
+    // each pass looks its page up once.  The loads of a fetch are unconditional (rows past the context
+    // or on an invalid page id read row `trow` of page 0 instead and are zeroed when they reach LDS).
     struct Staged {
         TileRegs<kTileKeys, kThreads> regs;
         unsigned row_ok;       // bit p: this thread's row of pass p holds a real key
