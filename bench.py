@@ -235,6 +235,13 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, maske
     dt = time.perf_counter() - t0
     done = sum(s.num_completion_tokens for s in seqs)
     st = eng.stats
+    # what the run must have done, whatever its speed: every sequence complete, no mask token left, one step-map
+    # entry per token, and (no confidence of a random-init model reaches the threshold) 8 denoising passes + 1
+    # caching pass per block, the first denoising pass of the first block being the prefill
+    blocks = new_tokens // S
+    assert all(s.num_completion_tokens == new_tokens and len(s.step_map) == new_tokens for s in seqs), "incomplete generation"
+    assert not any(cfg.mask_token_id in s.completion_token_ids for s in seqs), "mask token in the output"
+    assert st["decode_passes"] == blocks * (steps_per_block + 1) - 1, f"unexpected pass count {st['decode_passes']}"
     out = dict(tokens_per_s=round(done / dt, 1), seconds=round(dt, 3), committed_tokens=done, batch=batch,
                prefill_passes=st["prefill_passes"], decode_passes=st["decode_passes"],
                prefill_s=round(st["prefill_s"], 3), decode_s=round(st["decode_s"], 3),
