@@ -234,6 +234,28 @@ int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
 
 /*
+ * Top-k / top-p filtering of logits before sampling -- replaces top_k_logits and top_p_logits of the
+ * HF variant (mineru_diffusion/modeling_mineru_diffusion.py:585-600), applied in the order of
+ * sample_with_temperature_topk_topp (:608-611): out = logits with every element below the row's
+ * cut-off value set to -inf, to be passed on to mdx_confidence_argmax / mdx_unmask_step (whose noise
+ * input then samples from the filtered distribution as torch.multinomial does at :613).
+ *
+ * logits, out: [rows, vocab], MDX_BF16 or MDX_F16 (the cut-off is found by counting over the 65 536
+ * values a 16-bit element can take; MDX_F32 is refused), row strides in elements; out may be logits
+ * itself.  top_k = 0 (or >= vocab) switches the top-k filter off, top_p >= 1 the top-p filter.
+ * top-k keeps the elements >= the k-th largest value (equal values are all kept, as in the reference);
+ * top-p keeps, of what top-k kept and with probabilities softmax(kept / T), the elements >= the value at
+ * which the cumulative probability taken from the largest element down first exceeds top_p (the
+ * reference keeps that element too; among EQUAL values at the cut-off its sort order decides, here all
+ * of them are kept).  temperatures as for mdx_confidence_argmax.  No workspace.
+ */
+int mdx_filter_logits(const void* logits, int64_t row_stride, int32_t dtype,
+                      const float* temperatures, int32_t rows_per_temp,
+                      int32_t top_k, float top_p,
+                      void* out, int64_t out_row_stride,
+                      int64_t rows, int64_t vocab, mdx_stream_t stream);
+
+/*
  * Fused producer of the attention inputs for one decoder layer: per-head RMSNorm of q and k,
  * rotary embedding, and the KV-cache store, in one pass over the fused QKV projection output --
  * replaces the chain q_norm / k_norm / rotary_emb / store_kvcache of

@@ -292,6 +292,34 @@ def confidence_argmax(logits: torch.Tensor, temperatures: torch.Tensor | None = 
     return x0.view(lead), x0_p.view(lead)
 
 
+def filter_logits(logits: torch.Tensor, top_k: int = 0, top_p: float = 1.0,
+                  temperatures: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """top_k_logits then top_p_logits of the HF variant (modeling_mineru_diffusion.py:585-600, in the
+    order of :608-611) on bf16 / fp16 logits [..., V]: a copy (or `out`, which may be `logits`) with
+    every element below the row's cut-off set to -inf.  Feed the result to confidence_argmax /
+    unmask_step; their `noise` input (Gumbel) then samples from the filtered distribution.  top_k = 0
+    and top_p >= 1 switch the respective filter off.  temperatures as for confidence_argmax (they
+    enter the top-p probabilities only)."""
+    _need_gpu(logits, temperatures, out)
+    l2 = _logits2d(logits)
+    rows, vocab = l2.shape
+    if out is None:
+        out = torch.empty(logits.shape, dtype=logits.dtype, device=logits.device)
+    assert out.shape == logits.shape and out.dtype == logits.dtype
+    assert out.stride(-1) == 1, "out must have unit stride along the vocabulary"
+    o2 = out if out.dim() == 2 else out.view(-1, vocab)          # raises if that would need a copy
+    rows_per_temp, t_ptr = 1, None
+    if temperatures is not None:
+        temperatures = temperatures.reshape(-1).to(torch.float32).contiguous()
+        assert rows % temperatures.numel() == 0
+        rows_per_temp = rows // temperatures.numel()
+        t_ptr = temperatures.data_ptr()
+    rc = _lib.lib().mdx_filter_logits(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, rows_per_temp,
+                                      int(top_k), float(top_p), o2.data_ptr(), o2.stride(0), rows, vocab, _stream(logits))
+    check(rc, "filter_logits")
+    return out
+
+
 def select_transfer(x0: torch.Tensor, x0_p: torch.Tensor, tokens: torch.Tensor, mask_token_id: int,
                     threshold: float, k: int = 1):
     """Device form of the selection loop (sampler.py:32-54, modeling_mineru_diffusion.py:518-532).
@@ -310,10 +338,14 @@ def select_transfer(x0: torch.Tensor, x0_p: torch.Tensor, tokens: torch.Tensor, 
 
 
 def unmask_step(logits: torch.Tensor, tokens: torch.Tensor, mask_token_id: int, threshold: float, k: int = 1,
-                temperatures: torch.Tensor | None = None, noise: torch.Tensor | None = None):
+                temperatures: torch.Tensor | None = None, noise: torch.Tensor | None = None,
+                top_k: int = 0, top_p: float = 1.0):
     """One whole unmask step on the device: logits [bs, S, V], tokens [bs, S] int64 (in place).
-    Returns (x0, x0_p, transfer, count)."""
+    Returns (x0, x0_p, transfer, count).  top_k / top_p (off by default, as in
+    modeling_mineru_diffusion.py:602,633-634) put filter_logits in front of the step."""
     _need_gpu(logits, tokens, temperatures, noise)
+    if top_k > 0 or top_p < 1.0:
+        logits = filter_logits(logits, top_k, top_p, temperatures)
     assert tokens.dtype == torch.int64 and tokens.is_contiguous()
     bs, S = tokens.shape
     l2 = _logits2d(logits)

@@ -38,6 +38,38 @@ def confidence_argmax(logits: np.ndarray, temperatures=None, noise: np.ndarray |
     return x0, chosen / e.sum(axis=-1)
 
 
+def filter_logits(logits: np.ndarray, top_k: int = 0, top_p: float = 1.0, temperatures=None) -> np.ndarray:
+    """logits [rows, V] -> float64 copy with the filtered-out elements at -inf.
+
+    modeling_mineru_diffusion.py:608-611  top-k first (if top_k > 0), then top-p (if top_p < 1)
+    :585-590  top-k: elements below the k-th largest VALUE go (elements equal to it stay)
+    :593-600  top-p: sort descending, cumulative softmax; an element goes when the cumulative
+              probability BEFORE it already exceeds p (the crossing element stays, the first always)
+    :606      the probabilities are those of logits / T
+
+    Defined here where the reference leaves it open: among equal values at the top-p cut-off the
+    reference's (unstable) sort order decides which stay; here all of them stay, so both filters
+    are "keep x >= one value of the row".  temperatures: scalar or one per row."""
+    x = np.asarray(logits, dtype=np.float64)
+    rows, V = x.shape
+    T = np.ones(rows) if temperatures is None else np.broadcast_to(np.asarray(temperatures, dtype=np.float64).reshape(-1), (rows,))
+    out = x.copy()
+    for r in range(rows):
+        keep = np.ones(V, dtype=bool)
+        if 0 < top_k < V:
+            kth = np.sort(x[r])[V - top_k]
+            keep &= x[r] >= kth
+        if top_p < 1.0 and np.isfinite(x[r].max()):
+            kept = np.sort(x[r][keep])[::-1] / T[r]
+            pr = np.exp(kept - kept[0])
+            cum = np.cumsum(pr / pr.sum())
+            over = np.nonzero(cum > top_p)[0]
+            cut = kept[over[0]] if len(over) else kept[-1]
+            keep &= x[r] / T[r] >= cut
+        out[r, ~keep] = -np.inf
+    return out
+
+
 def select_transfer(conf: np.ndarray, masked: np.ndarray, threshold: float, k: int) -> np.ndarray:
     """conf [bs, S] float, masked [bs, S] bool -> transfer [bs, S] bool.
 

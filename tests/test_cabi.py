@@ -74,6 +74,12 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 0, one, one, 2, 32, null) == -1       # k < 1
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 1, one, one, 2, 2000, null) == -2      # block too long
     assert L.mdx_confidence_argmax(one, 10, 0, null, 1, null, 0, one, one, 4, 20, null, 0, null) == -2   # stride < vocab
+    fl = lambda **kw: L.mdx_filter_logits(one, kw.get("stride", 100), kw.get("dtype", 0), null, 1,           # noqa: E731
+                                          kw.get("k", 5), kw.get("p", 0.9), one, 100, kw.get("rows", 4), 100, null)
+    assert fl(dtype=2) == -2 and b"16-bit" in L.mdx_last_error()      # fp32 logits: the cut-off is found by counting 16-bit values
+    assert fl(k=-1) == -1 and fl(p=-0.5) == -1 and fl(p=float("nan")) == -1
+    assert fl(stride=50) == -2
+    assert fl(rows=0) == 0
     # the single-launch paged call: with about a pair per CU (32 sequences x 8 head groups) it needs the counters
     big = ctypes.c_void_p(1 << 20)
     ws32 = L.mdx_paged_block_attn_workspace_bytes(32, 32, 16, 8, 128, 17, 256)

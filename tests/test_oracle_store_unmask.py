@@ -139,3 +139,73 @@ def test_unmask_step_end_to_end_small():
     assert (new[0, :3] == [1, 2, 3]).all() and not tr[0, :3].any()
     assert (new[tr] == x0[tr]).all() and (new[~tr] == tokens[~tr]).all()
     assert tr.sum(-1).tolist() == [2, 2] or (p > 0.9).any()
+
+
+# ---- filter_logits (top-k / top-p before sampling) ----------------------------------------------
+
+def _torch_topk_topp(logits, k, p, T=1.0):
+    """The filters written with the library routines the reference composes them from (topk / where;
+    sort / softmax / cumsum / scatter), in fp64."""
+    x = torch.from_numpy(np.asarray(logits, dtype=np.float64)) / T
+    if k > 0:
+        kth = torch.topk(x, k).values[..., -1, None]
+        x = torch.where(x < kth, torch.full_like(x, float("-inf")), x)
+    if p < 1.0:
+        srt, order = torch.sort(x, descending=True)
+        drop = torch.cumsum(torch.softmax(srt, dim=-1), dim=-1) > p
+        drop = torch.cat([torch.zeros_like(drop[..., :1]), drop[..., :-1]], dim=-1)
+        x = x.masked_fill(torch.zeros_like(drop).scatter(-1, order, drop), float("-inf"))
+    return torch.isfinite(x).numpy()
+
+
+@pytest.mark.parametrize("k,p,T", [(5, 1.0, 1.0), (0, 0.9, 1.0), (0, 0.3, 0.7), (40, 0.8, 1.3), (1, 1.0, 1.0), (0, 0.0, 1.0), (200, 0.999, 1.0)])
+def test_filter_matches_library_formulation_on_tie_free_rows(k, p, T):
+    rng = np.random.default_rng(k * 7 + int(p * 100))
+    x = rng.permutation(np.linspace(-6, 9, 6 * 257)).reshape(6, 257)          # all values distinct
+    got = np.isfinite(oracle.filter_logits(x, top_k=k, top_p=p, temperatures=T))
+    assert np.array_equal(got, _torch_topk_topp(x, k, p, T))
+    kept = oracle.filter_logits(x, top_k=k, top_p=p, temperatures=T)
+    assert np.array_equal(kept[got], x[got])                                   # survivors keep their value
+
+
+def test_filter_counting_and_mass_invariants():
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 3, (16, 500))
+    for k in (1, 7, 499):
+        assert np.all(np.isfinite(oracle.filter_logits(x, top_k=k)).sum(1) == k)
+    assert np.array_equal(oracle.filter_logits(x, top_k=0, top_p=1.0), x)
+    assert np.array_equal(oracle.filter_logits(x, top_k=500), x)              # k >= V: nothing goes
+    for p in (0.1, 0.5, 0.95):
+        keep = np.isfinite(oracle.filter_logits(x, top_p=p))
+        pr = np.exp(x - x.max(1, keepdims=True))
+        pr /= pr.sum(1, keepdims=True)
+        for r in range(16):
+            mass = pr[r][keep[r]].sum()
+            assert mass > p and mass - pr[r][keep[r]].min() <= p               # minimal prefix that exceeds p
+            assert pr[r][keep[r]].min() > pr[r][~keep[r]].max()                # and it is a prefix
+
+
+def test_filter_brute_force_and_ties():
+    x = np.array([[2.0, -1.0, 0.5, 3.0, 0.0, 1.5, -2.0, 2.5]])
+    pr = np.exp(x[0]) / np.exp(x[0]).sum()
+    order = np.argsort(-x[0])
+    for p in np.linspace(0.01, 0.99, 50):
+        n = 1
+        while pr[order[:n]].sum() <= p:
+            n += 1
+        want = np.zeros(8, dtype=bool)
+        want[order[:n]] = True
+        assert np.array_equal(np.isfinite(oracle.filter_logits(x, top_p=float(p)))[0], want)
+    # top-k keeps every element equal to the k-th largest (`logits < min_values` drops none of them)
+    t = np.array([[1.0, 3.0, 2.0, 2.0, 2.0, 0.0]])
+    assert np.isfinite(oracle.filter_logits(t, top_k=2)).sum() == 4
+    assert np.array_equal(np.isfinite(oracle.filter_logits(t, top_k=2)), _torch_topk_topp(t, 2, 1.0))
+    # top-p: all elements equal to the crossing value stay (the reference's sort order would pick among them)
+    assert np.isfinite(oracle.filter_logits(t, top_p=0.6)).sum() == 4
+    # temperature enters the top-p probabilities: a colder row needs fewer elements
+    x2 = np.linspace(0, 5, 50)[None]
+    assert np.isfinite(oracle.filter_logits(x2, top_p=0.9, temperatures=0.5)).sum() < np.isfinite(oracle.filter_logits(x2, top_p=0.9, temperatures=2.0)).sum()
+    # rows already holding -inf: those never come back, and an all -inf row is left alone
+    y = np.array([[0.0, -np.inf, 1.0, -np.inf], [-np.inf] * 4])
+    f = oracle.filter_logits(y, top_k=3, top_p=0.99)
+    assert np.array_equal(np.isfinite(f), [[True, False, True, False], [False] * 4])
