@@ -349,7 +349,7 @@ int mdx_masked_rows(const int64_t* tokens, const int32_t* phase, int64_t mask_to
  * step, step += 1) and Scheduler.postprocess (engine/scheduler.py:65-82) per lane.  A denoising lane
  * whose block has no masked position left becomes caching; a caching lane (this pass has stored its
  * block's K/V) appends the block to out_tokens / out_steps [bs, out_stride] at offset lens - first_len
- * (Sequence.append_block, engine/sequence.py:97-101), adds block_len to lens, refills the block with
+ * (Sequence.append_block, engine/sequence.py:97-101; positions at or beyond out_stride are dropped), adds block_len to lens, refills the block with
  * mask_token_id and becomes idle if the block held one of its n_stop stop_ids [bs, n_stop] (-1 = unused
  * entry) or lens - first_len >= max_new, else denoising again.  status [bs, 4] int32 = (phase, lens,
  * masked positions left, positions committed by this pass).

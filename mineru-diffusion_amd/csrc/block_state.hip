@@ -126,8 +126,10 @@ __global__ __launch_bounds__(64) void block_advance_kernel(const AdvanceParams P
         const int done = len - P.first_len[b];
         for (int p = lane; p < S; p += 64) {
             const int64_t at = (int64_t)b * S + p;
-            P.out_tokens[(int64_t)b * P.out_stride + done + p] = P.tokens[at];
-            P.out_steps[(int64_t)b * P.out_stride + done + p] = P.step_map[at];   // written by this same lane above, if at all
+            if (done >= 0 && done + p < P.out_stride) {                           // a full output row drops the rest
+                P.out_tokens[(int64_t)b * P.out_stride + done + p] = P.tokens[at];
+                P.out_steps[(int64_t)b * P.out_stride + done + p] = P.step_map[at];   // written by this same lane above, if at all
+            }
             P.tokens[at] = P.mask_token_id;
         }
         len += S;

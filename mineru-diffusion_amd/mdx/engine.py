@@ -789,8 +789,12 @@ class BlockDiffusionEngine:
     def _device_pass(self, seqs) -> int:
         """Enqueues one decode pass of the device loop and, one pass late, looks at what the passes before it did."""
         g = self._loaded
+        moved = 0
         if g is None or g["seqs"] != seqs:
-            self._drain()
+            moved += self._drain() or 0
+            seqs = [s for s in seqs if not s.is_finished]   # the drain may have retired some of them
+            if not seqs:
+                return moved
             g = self._load_lanes(seqs)
         self._cover_pages(g)
         sp = seqs[0].sampling_params
@@ -807,14 +811,14 @@ class BlockDiffusionEngine:
         g["status_done"][slot].record()
         g["pending"].append(g["pass_no"])
         g["pass_no"] += 1
-        moved, finished = 0, False
+        finished = False
         keep = 1 if self.replay_ahead else 0               # passes that may stay unread while the next one is prepared
         while len(g["pending"]) > keep:
             n, fin = self._read_status(g, g["pending"].pop(0))
             moved += n
             finished |= fin
         if finished:
-            self._drain()
+            moved += self._drain() or 0
         return moved
 
     def step(self):                                        # llm_engine.py:66-73
@@ -828,6 +832,8 @@ class BlockDiffusionEngine:
             self.stats["prefill_s"] += time.perf_counter() - t0
             return n, True
         seqs = list(self.running)[:self.max_num_seqs]
+        if not seqs:
+            return 0, False
         n = None
         if self._device_loop_usable(seqs):
             try:
