@@ -200,7 +200,7 @@ def make_cfg4(dev, n_sets=2, seed=4):
 
 
 # ----------------------------------------------------------------------------- config 5
-def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, masked_rows_only=True):
+def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, masked_rows_only=True, gumbel_seed=None):
     """Random-init SDAR-shaped decoder (28 layers, hidden 2048, Hq 16 / Hkv 8 / d 128, SwiGLU 6144,
     vocab 151936), batch 32, 1024 random prefix embeddings + 64 prompt tokens per sequence, 2048 new
     tokens in 32-token blocks, k = 32/8 = 4 committed positions per denoising pass, threshold 0.9.
@@ -211,7 +211,7 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, maske
     model = Decoder(cfg, dev, seed=5)
     pages_per_seq = (1088 + new_tokens + PAGE - 1) // PAGE + 1
     eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5, decode_graphs=True, max_model_len=4096,
-                               masked_rows_only=masked_rows_only)
+                               masked_rows_only=masked_rows_only, gumbel_seed=gumbel_seed)
     g = torch.Generator().manual_seed(5)
     prompts = []
     for _ in range(batch):
@@ -377,7 +377,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-full-logits-leg", action="store_true",
                     help="decode leg: skip the second generation that projects all 32 positions of every block")
-    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,decode (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,decode (default all; gumbel and filter run inside unmask)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -542,6 +542,34 @@ def main():
             dtoks.copy_(fresh4)
         um_ms, um_min = time_kernel(unmask, W, K, graph=True, before_timed=remask)
         result_ops["unmask_step"] = op_entry(um_ms, um_min, "hbm", c4["bytes"], 1e6, PEAK_HBM_GBS, "GB/s")
+        if want("gumbel"):
+            # the reference's own sampling (sampler.py:15-18: Gumbel noise on every logit before the argmax), the noise
+            # drawn inside the kernel: bound by the generator's integer multiplies and the two logarithms per logit
+            def unmask_gumbel(i):
+                lg = c4["logits"][i % len(c4["logits"])]
+                dtok = dtoks[next(calls) % n_calls]
+                rc = L.mdx_unmask_step_gumbel(lg.data_ptr(), VOCAB, 0, None, 2024, i, None, None, dtok.data_ptr(), MASK_ID, 0.9, 4,
+                                              x0_4.data_ptr(), p_4.data_ptr(), tr_4.data_ptr(), cnt_4.data_ptr(), 32, S, VOCAB,
+                                              ws4.data_ptr(), ws_bytes4, raw_stream())
+                assert rc == 0
+            gm_ms, gm_min = time_kernel(unmask_gumbel, 2, max(3, K // 4), graph=True, before_timed=remask)
+            result_ops["unmask_step_gumbel"] = op_entry(gm_ms, gm_min, "hbm", c4["bytes"], 1e6, PEAK_HBM_GBS, "GB/s",
+                                                        dict(note="Gumbel noise drawn in the kernel (Philox-4x32-10 per 4 logits): compute-bound, "
+                                                                  "not a bandwidth figure; the same step with the noise made by torch ops and "
+                                                                  "passed as a tensor takes about 1 ms"))
+        if want("filter"):
+            # the HF variant's optional top-k / top-p filter in front of the step (off by default there): a filtered
+            # copy of the same logits, algorithmic bytes = one read + one write of them
+            flt_out = torch.empty_like(c4["logits"][0])
+
+            def logit_filter(i):
+                lg = c4["logits"][i % len(c4["logits"])]
+                rc = L.mdx_filter_logits(lg.data_ptr(), VOCAB, 0, None, 1, 50, 0.9, flt_out.data_ptr(), VOCAB, rows4, VOCAB, raw_stream())
+                assert rc == 0
+            fl_ms, fl_min = time_kernel(logit_filter, 2, max(3, K // 4), graph=True)
+            result_ops["filter_logits"] = op_entry(fl_ms, fl_min, "hbm", 2 * c4["bytes"], 1e6, PEAK_HBM_GBS, "GB/s",
+                                                   dict(top_k=50, top_p=0.9, note="off by default in the reference; reads each row four to five times"))
+            del flt_out
         del c4
         torch.cuda.empty_cache()
 
@@ -555,6 +583,8 @@ def main():
         if not args.no_full_logits_leg:
             full = run_cfg5(dev, masked_rows_only=False)
             decode["with_full_logits"] = {k: full[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass", "vocabulary_projection")}
+            noisy = run_cfg5(dev, gumbel_seed=5)
+            decode["with_gumbel_sampling"] = {k: noisy[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass")}
 
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
     cpu = None

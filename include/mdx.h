@@ -211,7 +211,9 @@ int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
  * Per sequence b (block length S <= 1024): masked = tokens[b,:] == mask_token_id;
  * conf = masked ? x0_p : -inf; hi = conf > threshold (strict).  If
  * count(hi) >= k commit all of hi, else commit the min(k, count(masked)) most
- * confident masked positions (ties: lower position first).  k = 1 gives the
+ * confident masked positions (ties: lower position first; a position whose
+ * x0_p is -inf is never committed, which lets a caller mark rows it has no
+ * fresh confidence for).  k = 1 gives the
  * engine's rule (sampler.py:41-50), k = block/steps the HF rule.  Writes
  * transfer[b,p] (uint8 0/1), tokens[b,p] = x0[b,p] where committed (in place),
  * and count[b] = number committed (int32).
@@ -232,6 +234,37 @@ int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
                     int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
                     int32_t bs, int32_t block_len, int64_t vocab,
                     void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+
+/*
+ * The same two calls with the Gumbel noise of Sampler.prepare (layers/sampler.py:15-16:
+ * gumbel = -log(Exponential(1)), added to logits / T before the argmax) drawn inside the kernel
+ * instead of read from a tensor.  The draw is a pure function of (seed, offset, row, column):
+ * Philox-4x32-10 with key = seed (low word, high word) and counter = (column / 4, row, offset low
+ * word, offset high word), whose four 32-bit outputs serve columns 4*(column/4) .. +3; an output r
+ * becomes u = ((r >> 9) + 1/2) / 2^23 and the noise is -ln(-ln u).  A caller gives every step
+ * another offset (as it would advance a generator); offset_dev, when not NULL, points to an int64
+ * on the device whose value is added to offset when the kernel runs, so that a replayed HIP graph
+ * can step it; row_ids, when not NULL, gives per logits row the row coordinate to use (int64
+ * [rows], on the device; values below 2^32), so that a caller who compacted its rows keeps the noise of the
+ * uncompacted layout.  x0_p is the softmax of logits / T at the drawn token (without noise), as in
+ * sampler.py:20-21.  mdx_gumbel_noise writes the noise tensor that these calls stand for
+ * ([rows <= 65535, vocab] fp32): mdx_confidence_argmax with that tensor gives the same bits.
+ */
+int mdx_confidence_argmax_gumbel(const void* logits, int64_t row_stride, int32_t dtype,
+                                 const float* temperatures, int32_t rows_per_temp,
+                                 uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                                 int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
+                                 void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+int mdx_unmask_step_gumbel(const void* logits, int64_t row_stride, int32_t dtype,
+                           const float* temperatures,
+                           uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                           int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                           int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                           int32_t bs, int32_t block_len, int64_t vocab,
+                           void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+int mdx_gumbel_noise(float* noise, int64_t noise_row_stride, int64_t rows, int64_t vocab,
+                     uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                     mdx_stream_t stream);
 
 /*
  * Top-k / top-p filtering of logits before sampling -- replaces top_k_logits and top_p_logits of the

@@ -28,11 +28,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 template <typename T> struct Bits16;
 template <> struct Bits16<__bf16> {
-    static constexpr uint32_t kNegInf = 0xff80u, kMaxFinite = 0x7f7fu;
+    static constexpr uint32_t kNegInf = 0xff80u;
     static __device__ __forceinline__ float value(uint32_t b) { return __uint_as_float(b << 16); }
 };
 template <> struct Bits16<__half> {
-    static constexpr uint32_t kNegInf = 0xfc00u, kMaxFinite = 0x7bffu;
+    static constexpr uint32_t kNegInf = 0xfc00u;
     static __device__ __forceinline__ float value(uint32_t b) { return __half2float(__ushort_as_half((unsigned short)b)); }
 };
 

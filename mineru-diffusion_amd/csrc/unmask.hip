@@ -141,13 +141,72 @@ __device__ __forceinline__ void visit(Partial& p, float x, int index, float c, f
     }
 }
 
+// --- Gumbel noise drawn in the kernel ------------------------------------------------------------
+// Sampler.prepare draws gumbel = -log(Exponential(1)) per logit (sampler.py:15-16).  Here the draw is
+// a pure function of (seed, offset, row, column): Philox-4x32-10 (Salmon et al., "Parallel random
+// numbers: as easy as 1, 2, 3", 2011) with key = seed and counter = (column / 4, row, offset), whose
+// four 32-bit outputs serve columns 4*(column/4) .. +3.  So the noise does not depend on the launch
+// geometry, a caller reproduces a step from three integers, and nothing is read from memory.
+struct NoiseSpec {
+    const float* noise; int64_t noise_row_stride;      // explicit noise tensor, or
+    bool philox; uint32_t key0, key1;                   // noise from the generator: seed,
+    uint64_t offset; const int64_t* offset_dev;         // offset (+ *offset_dev when given: a counter a graph replay can advance),
+    const int64_t* row_ids;                             // and the row coordinate of each logits row (NULL: the row's own index)
+};
+
+struct U4 { uint32_t x, y, z, w; };
+
+__device__ __forceinline__ U4 philox4x32_10(U4 c, uint32_t k0, uint32_t k1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c.x), lo0 = 0xD2511F53u * c.x;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c.z), lo1 = 0xCD9E8D57u * c.z;
+        c = U4{hi1 ^ c.y ^ k0, lo1, hi0 ^ c.w ^ k1, lo0};
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return c;
+}
+
+// 32 random bits -> u = (top 23 bits + 1/2) / 2^23 in (0, 1) -> e = -ln u (a unit exponential) -> -ln e.
+// Next to u = 1 the logarithm loses its relative accuracy, and those are the draws that win an argmax:
+// there e comes from the series of -ln(1 - w), w = 1 - u (exact in fp32).
+__device__ __forceinline__ float gumbel_of(uint32_t bits) {
+    constexpr float kLn2 = 0.69314718055994531f;
+    const float k = (float)(bits >> 9);
+    const float u = (k + 0.5f) * 1.1920928955078125e-07f;                    // 2^-23
+    const float w = (8388607.5f - k) * 1.1920928955078125e-07f;              // 1 - u
+    const float series = w * (1.0f + w * (0.5f + w * (0.33333334f + w * 0.25f)));
+    const float e = w < 0.015625f ? series : -kLn2 * __builtin_amdgcn_logf(u);
+    return -kLn2 * __builtin_amdgcn_logf(e);
+}
+
+struct RowNoise {                       // the generator's coordinates of one logits row
+    uint32_t key0, key1, row, off_lo, off_hi;
+    __device__ __forceinline__ U4 group(uint32_t column_group) const {
+        return philox4x32_10(U4{column_group, row, off_lo, off_hi}, key0, key1);
+    }
+    __device__ __forceinline__ float at(int column) const {
+        const U4 r = group((uint32_t)column >> 2);
+        const uint32_t b[4] = {r.x, r.y, r.z, r.w};
+        return gumbel_of(b[column & 3]);
+    }
+};
+
+__device__ __forceinline__ RowNoise row_noise(const NoiseSpec& N, int64_t row) {
+    const uint64_t off = N.offset + (N.offset_dev ? (uint64_t)*N.offset_dev : 0ull);
+    const int64_t rid = N.row_ids ? N.row_ids[row] : row;
+    return RowNoise{N.key0, N.key1, (uint32_t)rid, (uint32_t)off, (uint32_t)(off >> 32)};
+}
+
 // grid = (rows, nsplit).  Each workgroup reduces chunks [split*cps, (split+1)*cps)
 // of one row; split 0 also takes the unaligned head and tail elements.
-template <typename T, bool NOISE>
+// NOISE: 0 = plain argmax, 1 = noise read from a tensor, 2 = noise drawn in the kernel.
+template <typename T, int NOISE>
 __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
     const T* __restrict__ logits, int64_t row_stride,
     const float* __restrict__ temperatures, int rows_per_temp,
-    const float* __restrict__ noise, int64_t noise_row_stride,
+    const NoiseSpec N,
     int64_t vocab, int nsplit,
     Partial* __restrict__ partials,          // [rows, nsplit] when nsplit > 1
     int64_t* __restrict__ x0, float* __restrict__ x0_p)
@@ -157,7 +216,7 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
     const int split = blockIdx.y;
     const int tid = threadIdx.x;
     const T* rp = logits + row * row_stride;
-    const float* np = NOISE ? noise + row * noise_row_stride : nullptr;
+    const float* np = NOISE == 1 ? N.noise + row * N.noise_row_stride : nullptr;
     const float T_ = temperatures ? temperatures[row / rows_per_temp] : 1.0f;
     const float c = kLog2e / T_;
 
@@ -177,38 +236,48 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
     Partial p;
     p.m = kNegBig; p.s = 0.f; p.idx = kNoIndex; p.pick = kNegBig; p.pick_x = 0.f; p.pick_idx = kNoIndex;
 
-    if (!NOISE) {
-        // Per lane: running max m, h = -(m * c) rounded to fp32, and s = sum of exp2(x * c + h), each
-        // exponent one FMA (x * c + h is rounded once, so the term of x == m is exp2(lo) with
-        // lo = m * c + h, the rounding error of the product, known exactly).  The sum that the row
-        // reduction wants, sum of exp2((x - m) * c), is s * exp2(-lo): applied once per lane after
-        // the loop.  Folding m * c into the FMA without that correction would carry its rounding,
-        // 2^-24 |m c|, into every term (1e-3 at logits of thousands).
-        float m = kNegBig, s = 0.f, h = 0.f;
-        int first_at = -1;           // element (counted from the first aligned chunk) that first held m
+    // Softmax over 16-byte chunks (modes 0 and 2).  Per lane: running max m, h = -(m * c) rounded to fp32,
+    // and s = sum of exp2(x * c + h), each exponent one FMA (x * c + h is rounded once, so the term of x == m is exp2(lo) with
+    // lo = m * c + h, the rounding error of the product, known exactly).  The sum that the row
+    // reduction wants, sum of exp2((x - m) * c), is s * exp2(-lo): applied once per lane after
+    // the loop.  Folding m * c into the FMA without that correction would carry its rounding,
+    // 2^-24 |m c|, into every term (1e-3 at logits of thousands).
+    float m = kNegBig, s = 0.f, h = 0.f;
+    int first_at = -1;           // element (counted from the first aligned chunk) that first held m
+    auto take_values = [&](const float (&x)[EPC], int64_t chunk) {
+        float cm = x[EPC - 1];
+#pragma unroll
+        for (int i = 0; i + 2 < EPC; i += 2) cm = max3(cm, x[i], x[i + 1]);
+        if (EPC % 2 == 0) cm = max3(cm, x[EPC - 2], x[EPC - 2]);
+        if (cm > m) {
+            // found here, while the chunk is in registers: reading it again at the end
+            // would fetch a whole cache line per lane from HBM (10 % more traffic)
+            int j = EPC - 1;
+#pragma unroll
+            for (int i = EPC - 2; i >= 0; --i) if (x[i] == cm) j = i;
+            first_at = (int)chunk * EPC + j;
+            const float h_new = -(cm * c);
+            s = s > 0.f ? s * fast_exp2(h_new - h) : 0.f;   // h_new <= h once a finite maximum exists
+            m = cm;
+            h = h_new;
+        }
+        float acc = fast_exp2(__builtin_fmaf(x[0], c, h));
+#pragma unroll
+        for (int i = 1; i < EPC; ++i) acc += fast_exp2(__builtin_fmaf(x[i], c, h));
+        s += acc;
+    };
+    auto lane_softmax_done = [&]() {
+        if (m > kNegBig) s *= fast_exp2(-__builtin_fmaf(m, c, h));   // to the base of m itself (a lane that saw no finite element keeps s == 0)
+        p.m = m;
+        p.s = s;
+        if (first_at >= 0) p.idx = (int)lead + first_at;
+    };
+
+    if (NOISE == 0) {
         auto take = [&](const u32x4 u, int64_t chunk) {
             float x[EPC];
             Elem<T>::unpack(u, x);
-            float cm = x[EPC - 1];
-#pragma unroll
-            for (int i = 0; i + 2 < EPC; i += 2) cm = max3(cm, x[i], x[i + 1]);
-            if (EPC % 2 == 0) cm = max3(cm, x[EPC - 2], x[EPC - 2]);
-            if (cm > m) {
-                // found here, while the chunk is in registers: reading it again at the end
-                // would fetch a whole cache line per lane from HBM (10 % more traffic)
-                int j = EPC - 1;
-#pragma unroll
-                for (int i = EPC - 2; i >= 0; --i) if (x[i] == cm) j = i;
-                first_at = (int)chunk * EPC + j;
-                const float h_new = -(cm * c);
-                s = s > 0.f ? s * fast_exp2(h_new - h) : 0.f;   // h_new <= h once a finite maximum exists
-                m = cm;
-                h = h_new;
-            }
-            float acc = fast_exp2(__builtin_fmaf(x[0], c, h));
-#pragma unroll
-            for (int i = 1; i < EPC; ++i) acc += fast_exp2(__builtin_fmaf(x[i], c, h));
-            s += acc;
+            take_values(x, chunk);
         };
         int64_t ch = cbeg + tid;
         // Main loop: the next group's kUnroll loads are issued before this group is reduced, so a lane
@@ -238,27 +307,64 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
             }
         }
         for (; ch < cend; ch += kThreads) take(__builtin_nontemporal_load(cp + ch), ch);
-        if (m > kNegBig) s *= fast_exp2(-__builtin_fmaf(m, c, h));   // to the base of m itself (a lane that saw no finite element keeps s == 0)
-        p.m = m;
-        p.s = s;
-        if (first_at >= 0) p.idx = (int)lead + first_at;
+        lane_softmax_done();
         if (split == 0) {            // unaligned head and tail, a handful of elements
             for (int64_t e = tid; e < lead; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
             for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
         }
-    } else {
+    } else if (NOISE == 1) {
         // Noise path: 4 more bytes per element and a true division; element-wise.
         const int64_t ebeg = (split == 0) ? 0 : lead + cbeg * EPC;
         const int64_t eend = (split == nsplit - 1) ? vocab : lead + cend * EPC;
         for (int64_t e = ebeg + tid; e < eend; e += kThreads)
             visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, np[e]);
+    } else {
+        // Noise from the generator.  The softmax runs over 16-byte chunks as without noise; the noisy argmax is
+        // the arithmetic of the tensor path element by element (l = x / T by a true division, v = l + g, the
+        // larger v or at equal v the lower index wins), so both paths draw the same tokens.  A chunk whose first
+        // column is a multiple of 4 (every row that starts on a 16-byte boundary) takes whole generator
+        // outputs, EPC / 4 of them; otherwise every element asks for its own.
+        const RowNoise rn = row_noise(N, row);
+        const bool whole_groups = (lead & 3) == 0;
+        const bool unit_T = T_ == 1.0f;                 // x / 1 == x: the division is skipped, not approximated
+        float best = kNegBig, best_x = 0.f;
+        int best_idx = kNoIndex;
+        auto offer = [&](float x, int index, float g) {
+            const float v = (unit_T ? x : x / T_) + g;
+            if (v > best || (v == best && index < best_idx)) { best = v; best_x = x; best_idx = index; }
+        };
+        for (int64_t ch = cbeg + tid; ch < cend; ch += kThreads) {
+            float x[EPC];
+            Elem<T>::unpack(__builtin_nontemporal_load(cp + ch), x);
+            take_values(x, ch);
+            const int c0 = (int)(lead + ch * EPC);
+            if (whole_groups) {
+#pragma unroll
+                for (int q = 0; q < EPC / 4; ++q) {
+                    const U4 r = rn.group((uint32_t)(c0 >> 2) + q);
+                    offer(x[4 * q + 0], c0 + 4 * q + 0, gumbel_of(r.x));
+                    offer(x[4 * q + 1], c0 + 4 * q + 1, gumbel_of(r.y));
+                    offer(x[4 * q + 2], c0 + 4 * q + 2, gumbel_of(r.z));
+                    offer(x[4 * q + 3], c0 + 4 * q + 3, gumbel_of(r.w));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) offer(x[i], c0 + i, rn.at(c0 + i));
+            }
+        }
+        lane_softmax_done();
+        p.pick = best; p.pick_x = best_x; p.pick_idx = best_idx;
+        if (split == 0) {
+            for (int64_t e = tid; e < lead; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, rn.at((int)e));
+            for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, rn.at((int)e));
+        }
     }
 
     // Wavefront reduction, then across the workgroup's wavefronts through LDS.
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
-        const Partial o = shfl_xor(p, off, NOISE);
-        combine(p, o, c, NOISE);
+        const Partial o = shfl_xor(p, off, NOISE != 0);
+        combine(p, o, c, NOISE != 0);
     }
     __shared__ Partial wave_part[kThreads / mdx::kWave];
     if ((tid & (mdx::kWave - 1)) == 0) wave_part[tid / mdx::kWave] = p;
@@ -266,12 +372,12 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
     if (tid == 0) {
         Partial r = wave_part[0];
 #pragma unroll
-        for (int w = 1; w < kThreads / mdx::kWave; ++w) combine(r, wave_part[w], c, NOISE);
+        for (int w = 1; w < kThreads / mdx::kWave; ++w) combine(r, wave_part[w], c, NOISE != 0);
         if (nsplit > 1) {
             partials[row * nsplit + split] = r;
         } else {
             int64_t tok; float conf;
-            finish_row<NOISE>(r, c, tok, conf);
+            finish_row<(NOISE != 0)>(r, c, tok, conf);
             x0[row] = tok;
             x0_p[row] = conf;
         }
@@ -349,7 +455,7 @@ __global__ __launch_bounds__(kMaxBlockLen) void select_transfer_kernel(
                 rank += (cj > conf || (cj == conf && j < p)) ? 1 : 0;
             }
         }
-        commit = masked && rank < k;     // at most min(k, n_masked) positions
+        commit = masked && rank < k && conf > -INFINITY;     // at most min(k, n_masked) positions; a confidence of -inf is never committed
     }
     if (on) {
         transfer[at] = commit ? 1 : 0;
@@ -407,7 +513,7 @@ __global__ __launch_bounds__(mdx::kWave) void select_transfer_wave_kernel(
             const float cj = __shfl(conf, j);
             rank += (cj > conf || (cj == conf && j < p)) ? 1 : 0;
         }
-        commit = masked && rank < k;     // at most min(k, #masked) positions
+        commit = masked && rank < k && conf > -INFINITY;     // at most min(k, #masked) positions; a confidence of -inf is never committed
     }
     const int n_commit = __popcll(__ballot(commit));
     if (on) {
@@ -455,24 +561,52 @@ int pick_nsplit(int64_t rows, int64_t vocab) {
 
 template <typename T>
 int launch_confidence(const void* logits, int64_t row_stride, const float* temperatures, int rows_per_temp,
-                      const float* noise, int64_t noise_row_stride, int64_t* x0, float* x0_p,
+                      const NoiseSpec& N, int64_t* x0, float* x0_p,
                       int64_t rows, int64_t vocab, int nsplit, Partial* partials, bool finalize, hipStream_t stream)
 {
     const dim3 grid((unsigned)rows, (unsigned)nsplit);
-    if (noise)
-        confidence_argmax_kernel<T, true><<<grid, kThreads, 0, stream>>>(
-            (const T*)logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, vocab, nsplit, partials, x0, x0_p);
+    const bool noisy = N.noise != nullptr || N.philox;
+    if (N.philox)
+        confidence_argmax_kernel<T, 2><<<grid, kThreads, 0, stream>>>(
+            (const T*)logits, row_stride, temperatures, rows_per_temp, N, vocab, nsplit, partials, x0, x0_p);
+    else if (N.noise)
+        confidence_argmax_kernel<T, 1><<<grid, kThreads, 0, stream>>>(
+            (const T*)logits, row_stride, temperatures, rows_per_temp, N, vocab, nsplit, partials, x0, x0_p);
     else
-        confidence_argmax_kernel<T, false><<<grid, kThreads, 0, stream>>>(
-            (const T*)logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, vocab, nsplit, partials, x0, x0_p);
+        confidence_argmax_kernel<T, 0><<<grid, kThreads, 0, stream>>>(
+            (const T*)logits, row_stride, temperatures, rows_per_temp, N, vocab, nsplit, partials, x0, x0_p);
     int rc = mdx::check_launch("confidence_argmax");
     if (rc != MDX_OK || nsplit == 1 || !finalize) return rc;
     const unsigned fgrid = (unsigned)((rows + kThreads - 1) / kThreads);
-    if (noise)
+    if (noisy)
         confidence_finalize_kernel<true><<<fgrid, kThreads, 0, stream>>>(partials, nsplit, temperatures, rows_per_temp, rows, x0, x0_p);
     else
         confidence_finalize_kernel<false><<<fgrid, kThreads, 0, stream>>>(partials, nsplit, temperatures, rows_per_temp, rows, x0, x0_p);
     return mdx::check_launch("confidence_finalize");
+}
+
+// The noise tensor that the generator stands for, written out: [rows, vocab] fp32.
+__global__ __launch_bounds__(kThreads) void gumbel_noise_kernel(float* __restrict__ out, int64_t out_row_stride, int64_t vocab, const NoiseSpec N)
+{
+    const int64_t row = blockIdx.y;
+    const RowNoise rn = row_noise(N, row);
+    const int64_t group = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (group * 4 >= vocab) return;
+    const U4 r = rn.group((uint32_t)group);
+    const uint32_t b[4] = {r.x, r.y, r.z, r.w};
+    float* dst = out + row * out_row_stride + group * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (group * 4 + i < vocab) dst[i] = gumbel_of(b[i]);
+}
+
+NoiseSpec no_noise() { return NoiseSpec{nullptr, 0, false, 0, 0, 0, nullptr, nullptr}; }
+NoiseSpec tensor_noise(const float* noise, int64_t stride) { NoiseSpec n = no_noise(); n.noise = noise; n.noise_row_stride = stride; return n; }
+NoiseSpec generator_noise(uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids) {
+    NoiseSpec n = no_noise();
+    n.philox = true; n.key0 = (uint32_t)seed; n.key1 = (uint32_t)(seed >> 32);
+    n.offset = offset; n.offset_dev = offset_dev; n.row_ids = row_ids;
+    return n;
 }
 
 }  // namespace
@@ -487,7 +621,7 @@ namespace {
 
 int confidence_pass(const void* logits, int64_t row_stride, int32_t dtype,
                     const float* temperatures, int32_t rows_per_temp,
-                    const float* noise, int64_t noise_row_stride,
+                    const NoiseSpec& N,
                     int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
                     void* workspace, int64_t workspace_bytes, bool finalize, int* nsplit_out, hipStream_t stream)
 {
@@ -500,7 +634,7 @@ int confidence_pass(const void* logits, int64_t row_stride, int32_t dtype,
                 "confidence_argmax: rows %lld or vocab %lld out of range", (long long)rows, (long long)vocab);
     MDX_REQUIRE(row_stride >= vocab, MDX_EUNSUPPORTED, "confidence_argmax: row_stride %lld < vocab %lld", (long long)row_stride, (long long)vocab);
     MDX_REQUIRE(!temperatures || rows_per_temp > 0, MDX_EINVAL, "confidence_argmax: rows_per_temp must be positive");
-    MDX_REQUIRE(!noise || noise_row_stride >= vocab, MDX_EINVAL, "confidence_argmax: noise_row_stride < vocab");
+    MDX_REQUIRE(!N.noise || N.noise_row_stride >= vocab, MDX_EINVAL, "confidence_argmax: noise_row_stride < vocab");
     const int esz = dtype == MDX_F32 ? 4 : 2;
     MDX_REQUIRE((reinterpret_cast<uintptr_t>(logits) % esz) == 0, MDX_EUNSUPPORTED, "confidence_argmax: logits not element-aligned");
     const int nsplit = pick_nsplit(rows, vocab);
@@ -510,9 +644,9 @@ int confidence_pass(const void* logits, int64_t row_stride, int32_t dtype,
                 "confidence_argmax: workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
     Partial* partials = static_cast<Partial*>(workspace);
     switch (dtype) {
-        case MDX_BF16: return launch_confidence<__bf16>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
-        case MDX_F16:  return launch_confidence<__half>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
-        case MDX_F32:  return launch_confidence<float>(logits, row_stride, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
+        case MDX_BF16: return launch_confidence<__bf16>(logits, row_stride, temperatures, rows_per_temp, N, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
+        case MDX_F16:  return launch_confidence<__half>(logits, row_stride, temperatures, rows_per_temp, N, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
+        case MDX_F32:  return launch_confidence<float>(logits, row_stride, temperatures, rows_per_temp, N, x0, x0_p, rows, vocab, nsplit, partials, finalize, stream);
         default: return mdx::fail(MDX_EUNSUPPORTED, "confidence_argmax: dtype %d", dtype);
     }
 }
@@ -525,8 +659,34 @@ extern "C" int mdx_confidence_argmax(const void* logits, int64_t row_stride, int
                                      int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
                                      void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
 {
-    return confidence_pass(logits, row_stride, dtype, temperatures, rows_per_temp, noise, noise_row_stride, x0, x0_p,
+    return confidence_pass(logits, row_stride, dtype, temperatures, rows_per_temp, tensor_noise(noise, noise_row_stride), x0, x0_p,
                            rows, vocab, workspace, workspace_bytes, true, nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mdx_confidence_argmax_gumbel(const void* logits, int64_t row_stride, int32_t dtype,
+                                            const float* temperatures, int32_t rows_per_temp,
+                                            uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                                            int64_t* x0, float* x0_p, int64_t rows, int64_t vocab,
+                                            void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    return confidence_pass(logits, row_stride, dtype, temperatures, rows_per_temp, generator_noise(seed, offset, offset_dev, row_ids),
+                           x0, x0_p, rows, vocab, workspace, workspace_bytes, true, nullptr, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mdx_gumbel_noise(float* noise, int64_t noise_row_stride, int64_t rows, int64_t vocab,
+                                uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                                mdx_stream_t stream)
+{
+    MDX_REQUIRE(rows >= 0 && vocab >= 0, MDX_EINVAL, "gumbel_noise: negative size");
+    if (rows == 0 || vocab == 0) return MDX_OK;
+    MDX_REQUIRE(noise, MDX_EINVAL, "gumbel_noise: null pointer");
+    MDX_REQUIRE(noise_row_stride >= vocab, MDX_EINVAL, "gumbel_noise: noise_row_stride < vocab");
+    MDX_REQUIRE(vocab < (int64_t)0x7fffffff && rows <= 65535, MDX_EUNSUPPORTED,
+                "gumbel_noise: rows %lld (max 65535) or vocab %lld out of range", (long long)rows, (long long)vocab);
+    const dim3 grid((unsigned)(((vocab + 3) / 4 + kThreads - 1) / kThreads), (unsigned)rows);
+    gumbel_noise_kernel<<<grid, kThreads, 0, static_cast<hipStream_t>(stream)>>>(noise, noise_row_stride, vocab,
+                                                                                 generator_noise(seed, offset, offset_dev, row_ids));
+    return mdx::check_launch("gumbel_noise");
 }
 
 extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t* tokens,
@@ -544,24 +704,53 @@ extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t
                          transfer, count, bs, block_len, stream);
 }
 
-extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
-                               const float* temperatures, const float* noise, int64_t noise_row_stride,
-                               int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
-                               int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
-                               int32_t bs, int32_t block_len, int64_t vocab,
-                               void* workspace, int64_t workspace_bytes, mdx_stream_t stream_)
+namespace {
+
+int unmask_step_impl(const void* logits, int64_t row_stride, int32_t dtype,
+                     const float* temperatures, const NoiseSpec& N,
+                     int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                     int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                     int32_t bs, int32_t block_len, int64_t vocab,
+                     void* workspace, int64_t workspace_bytes, hipStream_t stream)
 {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && block_len >= 0, MDX_EINVAL, "unmask_step: negative size");
     MDX_REQUIRE(k >= 1, MDX_EINVAL, "unmask_step: k %d < 1", k);
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "unmask_step: block_len %d > %d", block_len, kMaxBlockLen);
     if (bs == 0 || block_len == 0) return MDX_OK;
     MDX_REQUIRE(tokens && transfer && count, MDX_EINVAL, "unmask_step: null pointer");
     // Without noise the selection kernel merges the row splits itself (one launch fewer).
+    const bool noisy = N.noise != nullptr || N.philox;
     int nsplit = 1;
-    int rc = confidence_pass(logits, row_stride, dtype, temperatures, block_len, noise, noise_row_stride,
-                             x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, noise != nullptr, &nsplit, stream);
+    int rc = confidence_pass(logits, row_stride, dtype, temperatures, block_len, N,
+                             x0, x0_p, (int64_t)bs * block_len, vocab, workspace, workspace_bytes, noisy, &nsplit, stream);
     if (rc != MDX_OK) return rc;
-    return launch_select(x0, x0_p, tokens, (nsplit > 1 && !noise) ? static_cast<const Partial*>(workspace) : nullptr, nsplit, temperatures,
+    return launch_select(x0, x0_p, tokens, (nsplit > 1 && !noisy) ? static_cast<const Partial*>(workspace) : nullptr, nsplit, temperatures,
                          mask_token_id, threshold, k, transfer, count, bs, block_len, stream);
+}
+
+}  // namespace
+
+extern "C" int mdx_unmask_step(const void* logits, int64_t row_stride, int32_t dtype,
+                               const float* temperatures, const float* noise, int64_t noise_row_stride,
+                               int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                               int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                               int32_t bs, int32_t block_len, int64_t vocab,
+                               void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    return unmask_step_impl(logits, row_stride, dtype, temperatures, tensor_noise(noise, noise_row_stride), tokens, mask_token_id,
+                            threshold, k, x0, x0_p, transfer, count, bs, block_len, vocab, workspace, workspace_bytes,
+                            static_cast<hipStream_t>(stream));
+}
+
+extern "C" int mdx_unmask_step_gumbel(const void* logits, int64_t row_stride, int32_t dtype,
+                                      const float* temperatures,
+                                      uint64_t seed, uint64_t offset, const int64_t* offset_dev, const int64_t* row_ids,
+                                      int64_t* tokens, int64_t mask_token_id, float threshold, int32_t k,
+                                      int64_t* x0, float* x0_p, uint8_t* transfer, int32_t* count,
+                                      int32_t bs, int32_t block_len, int64_t vocab,
+                                      void* workspace, int64_t workspace_bytes, mdx_stream_t stream)
+{
+    return unmask_step_impl(logits, row_stride, dtype, temperatures, generator_noise(seed, offset, offset_dev, row_ids), tokens,
+                            mask_token_id, threshold, k, x0, x0_p, transfer, count, bs, block_len, vocab, workspace, workspace_bytes,
+                            static_cast<hipStream_t>(stream));
 }

@@ -2,7 +2,7 @@
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int32, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int32, c_int64, c_uint64, c_void_p
 from pathlib import Path
 
 _HERE = Path(__file__).resolve().parent
@@ -19,7 +19,7 @@ def library_path() -> Path:
 
 
 # name -> (restype, argtypes); mirrors include/mdx.h one to one
-_P, _I32, _I64, _F = c_void_p, c_int32, c_int64, c_float
+_P, _I32, _I64, _F, _U64 = c_void_p, c_int32, c_int64, c_float, c_uint64
 SIGNATURES = {
     "mdx_version": (c_int32, []),
     "mdx_last_error": (c_char_p, []),
@@ -35,6 +35,10 @@ SIGNATURES = {
     "mdx_paged_block_attn_static": (c_int32, [_P, _P, _P, _P] + [_I64] * 9 + [_P, _I64, _P] + [_I32] * 7 + [_I64, _F, _I32, _P]),
     "mdx_confidence_argmax_workspace_bytes": (c_int64, [_I64, _I64]),
     "mdx_confidence_argmax": (c_int32, [_P, _I64, _I32, _P, _I32, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _P]),
+    "mdx_confidence_argmax_gumbel": (c_int32, [_P, _I64, _I32, _P, _I32, _U64, _U64, _P, _P, _P, _P, _I64, _I64, _P, _I64, _P]),
+    "mdx_unmask_step_gumbel": (c_int32, [_P, _I64, _I32, _P, _U64, _U64, _P, _P, _P, _I64, _F, _I32, _P, _P, _P, _P,
+                                         _I32, _I32, _I64, _P, _I64, _P]),
+    "mdx_gumbel_noise": (c_int32, [_P, _I64, _I64, _I64, _U64, _U64, _P, _P, _P]),
     "mdx_select_transfer": (c_int32, [_P, _P, _P, _I64, _F, _I32, _P, _P, _I32, _I32, _P]),
     "mdx_qk_norm_rope_store": (c_int32, [_P, _I64, _P, _P, _F, _P, _P, _I64, _P, _P, _I64, _P, _I64, _P, _P, _P, _I64,
                                          _I64, _I32, _I32, _I32, _I32, _P]),

@@ -330,8 +330,10 @@ class BlockDiffusionEngine:
         self.decode_graphs = decode_graphs                 # decode through the device loop (HIP graphs per batch size)
         self.max_model_len = max_model_len
         # Gumbel noise on the scaled logits before the argmax, as Sampler.prepare draws it (sampler.py:15-18);
-        # None = plain argmax (reproducible), an int seeds a device generator (reproducible per seed)
-        self.gumbel = None if gumbel_seed is None else torch.Generator(device=model.lm_head.device).manual_seed(gumbel_seed)
+        # None = plain argmax, an int seeds the generator inside the unmask kernel: the noise of a pass is a
+        # function of (seed, number of the sampling pass, row, column), so a seed reproduces a generation
+        self.gumbel_seed = gumbel_seed
+        self._rng_offset = 0                               # sampling passes so far: the generator offset of the next one
         self.replay_ahead = replay_ahead                   # device loop: enqueue pass p+1 before reading the status of pass p
         self.masked_rows_only = masked_rows_only           # device loop: logits for still-masked positions only
         self._graphs = {}                                  # captured batch size -> lane buffers and graphs
@@ -485,12 +487,6 @@ class BlockDiffusionEngine:
                     block_tables=self._block_tables(seqs), block_size=S)
         return ids.to(dev, non_blocking=True), pos.to(dev, non_blocking=True)
 
-    def _noise(self, logits):
-        if self.gumbel is None:
-            return None
-        e = torch.empty(logits.shape, dtype=torch.float32, device=logits.device).exponential_(generator=self.gumbel)
-        return -e.log_()
-
     def _temperatures(self, seqs):
         key = tuple(s.temperature for s in seqs)
         if self._temps is None or self._temps[0] != key:
@@ -502,7 +498,8 @@ class BlockDiffusionEngine:
         if sp.denoising_strategy != "low_confidence_dynamic":
             raise NotImplementedError(f"Denoising strategy {sp.denoising_strategy} not implemented")
         x = torch.stack([s.current_denoising_block for s in seqs]).to(self.device)
-        extra = {} if self.gumbel is None else {"noise": self._noise(logits)}
+        extra = {} if self.gumbel_seed is None else {"seed": self.gumbel_seed, "offset": self._rng_offset}
+        self._rng_offset += 1
         _, _, transfer, _n = self.unmask(logits, x, seqs[0].mask_token_id, sp.dynamic_threshold, sp.transfer_count,
                                          temperatures=self._temperatures(seqs), **extra)
         x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
@@ -552,7 +549,7 @@ class BlockDiffusionEngine:
         i32, i64, f32 = torch.int32, torch.int64, torch.float32
         fields = [("ids", i64, (gbs, S)), ("stop_ids", i64, (gbs, N_STOP)), ("step_map", i32, (gbs, S)), ("lens", i32, (gbs,)),
                   ("phase", i32, (gbs,)), ("step", i32, (gbs,)), ("first_len", i32, (gbs,)), ("max_new", i32, (gbs,)),
-                  ("temps", f32, (gbs,)), ("bt", i32, (gbs, width))]
+                  ("temps", f32, (gbs,)), ("rng_step", i64, (1,)), ("bt", i32, (gbs, width))]
         offsets, at = {}, 0
         for name, dt, shape in fields:
             offsets[name] = at
@@ -617,19 +614,30 @@ class BlockDiffusionEngine:
             _lib.check(_lib.lib().mdx_masked_rows(g["ids"].data_ptr(), g["phase"].data_ptr(), self.c.mask_token_id, gbs, S,
                                                   rows.data_ptr(), cap, g["n_rows"].data_ptr(), stream), "masked_rows")
             logits = F.linear(flat.index_select(0, rows), self.model.lm_head)
-            x0, p = confidence_argmax(logits, g["temps"].index_select(0, rows // S), self._noise(logits))
+            x0, p = confidence_argmax(logits, g["temps"].index_select(0, rows // S), **self._draw(g, rows))
             g["x0"].index_copy_(0, rows, x0)
             g["x0_p"].index_copy_(0, rows, p)
         else:
             logits = F.linear(flat, self.model.lm_head).view(gbs, S, -1)
-            x0, p = confidence_argmax(logits, g["temps"], self._noise(logits))
+            x0, p = confidence_argmax(logits, g["temps"], **self._draw(g, None))
             g["x0"].copy_(x0.view(-1))
             g["x0_p"].copy_(p.view(-1))
+
+    def _draw(self, g, rows):
+        """Generator arguments of a device-loop pass: the lanes' own pass counter as the offset, and for compacted
+        rows their places in the whole batch, so that compaction does not change the draw."""
+        if self.gumbel_seed is None:
+            return {}
+        return dict(seed=self.gumbel_seed, offset=0, offset_dev=g["rng_step"], row_ids=rows)
 
     def _head(self, g, cap: int, threshold: float, k: int):
         """The second half of a pass: logits of (at most) `cap` masked rows, the selection rule, and the advance of
         every lane's state (sampler.py:24-61 + scheduler.py:65-82 on the device)."""
         S, gbs = self.c.block_size, g["bs"]
+        if cap < gbs * S:
+            # rows that get no fresh logits in this pass (the host's bound `cap` fell short of the masked rows: a
+            # committed token that happens to be the mask token leaves its position masked) are not committed
+            g["x0_p"].fill_(float("-inf"))
         if cap > 0:
             self._logits_of_rows(g, cap)
         transfer, _count = select_transfer(g["x0"].view(gbs, S), g["x0_p"].view(gbs, S), g["ids"], self.c.mask_token_id, threshold, k)
@@ -639,6 +647,7 @@ class BlockDiffusionEngine:
             g["lens"].data_ptr(), g["first_len"].data_ptr(), g["max_new"].data_ptr(), g["stop_ids"].data_ptr(), N_STOP,
             g["out_tokens"].data_ptr(), g["out_steps"].data_ptr(), g["out_tokens"].stride(0), g["status"].data_ptr(),
             self.c.mask_token_id, gbs, S, stream), "block_advance")
+        g["rng_step"].add_(1)                               # the next pass draws other noise
 
     def _head_graph(self, g, cap, threshold, k):
         key = (cap, threshold, k)
@@ -674,6 +683,7 @@ class BlockDiffusionEngine:
         h["bt"].fill_(-1)
         h["stop_ids"].fill_(-1)
         h["ids"].fill_(mask)
+        h["rng_step"][0] = self._rng_offset
         for i, s in enumerate(seqs):
             h["ids"][i] = s.current_denoising_block
             h["step_map"][i] = s.current_step_map
@@ -719,9 +729,11 @@ class BlockDiffusionEngine:
             g["bt_copied"].record()
 
     def _rows_cap(self, g) -> int:
-        """An upper bound, known without asking the device, of the masked rows at the start of the pass about to be
-        enqueued, rounded up to an eighth of all rows: every denoising pass commits at least min(k, masked)
-        positions of a lane, a caching pass leaves a fresh block behind."""
+        """The number of rows that get logits in the pass about to be enqueued, rounded up to an eighth of all rows:
+        what the host, one pass behind, expects to be masked at most -- a denoising pass commits min(k, masked)
+        positions of a lane, a caching pass leaves a fresh block behind.  The expectation can fall short (a
+        committed token that is the mask token itself leaves its position masked); rows beyond it get no logits and
+        are not committed in that pass, and a denoising lane is never taken to be done before its status says so."""
         S, gbs = self.c.block_size, g["bs"]
         if not self.masked_rows_only:
             return gbs * S
@@ -732,7 +744,7 @@ class BlockDiffusionEngine:
             if ahead == 0:
                 bound += m if ph == DENOISING else 0
             else:
-                bound += S if ph == CACHING else max(0, m - k) if ph == DENOISING else 0
+                bound += S if ph == CACHING else max(1, m - k) if ph == DENOISING else 0
         step = max(1, gbs * S // 8)
         return min(gbs * S, -(-bound // step) * step)
 
@@ -799,13 +811,10 @@ class BlockDiffusionEngine:
         self._cover_pages(g)
         sp = seqs[0].sampling_params
         cap = self._rows_cap(g)
-        if self.gumbel is None:
-            head = self._head_graph(g, cap, float(sp.dynamic_threshold), int(sp.transfer_count))
-            g["fwd"].replay()
-            head.replay()
-        else:                                               # the noise comes from a generator: drawn eagerly, pass by pass
-            g["fwd"].replay()
-            self._head(g, cap, float(sp.dynamic_threshold), int(sp.transfer_count))
+        head = self._head_graph(g, cap, float(sp.dynamic_threshold), int(sp.transfer_count))
+        g["fwd"].replay()
+        head.replay()
+        self._rng_offset += 1
         slot = g["pass_no"] % 2
         g["status_host"][slot].copy_(g["status"], non_blocking=True)
         g["status_done"][slot].record()

@@ -43,18 +43,27 @@ class Sampler(nn.Module):
     selection); only the [bs, S] results cross to the host to update the Sequence objects.
 
     `k` is the number of positions committed when fewer than k exceed the threshold
-    (1 = the engine's rule, sampler.py:44-50).  `noise_fn(logits) -> fp32 noise` supplies the
-    Gumbel term of sampler.py:15-18 when sampling is wanted; None = plain argmax."""
+    (1 = the engine's rule, sampler.py:44-50).  The Gumbel term of sampler.py:15-18 comes from `seed`
+    (drawn inside the kernel by a counter-based generator; every call takes the next offset, so a seed
+    reproduces a run) or from `noise_fn(logits) -> fp32 noise`; neither = plain argmax."""
 
-    def __init__(self, k: int = 1, noise_fn=None):
+    def __init__(self, k: int = 1, noise_fn=None, seed: int | None = None):
         super().__init__()
+        assert noise_fn is None or seed is None, "either a noise function or a seed"
         self.k = k
         self.noise_fn = noise_fn
+        self.seed = seed
+        self.calls = 0                                      # the generator offset of the next call
+
+    def _noise_args(self, logits):
+        if self.seed is not None:
+            self.calls += 1
+            return dict(seed=self.seed, offset=self.calls - 1)
+        return dict(noise=self.noise_fn(logits) if self.noise_fn is not None else None)
 
     def prepare(self, logits: torch.Tensor, temperatures: torch.Tensor):
         from .ops import confidence_argmax
-        noise = self.noise_fn(logits) if self.noise_fn is not None else None
-        return confidence_argmax(logits, temperatures, noise)
+        return confidence_argmax(logits, temperatures, **self._noise_args(logits))
 
     def forward(self, logits: torch.Tensor, temperatures: torch.Tensor, seqs) -> int:
         strategy = seqs[0].sampling_params.denoising_strategy
@@ -62,9 +71,8 @@ class Sampler(nn.Module):
             raise NotImplementedError(f"Denoising strategy {strategy} not implemented")
         threshold = seqs[0].sampling_params.dynamic_threshold
         x = torch.stack([seq.current_denoising_block for seq in seqs], dim=0).to(logits.device)
-        noise = self.noise_fn(logits) if self.noise_fn is not None else None
         _, _, transfer, count = unmask_step(logits, x, seqs[0].mask_token_id, threshold, self.k,
-                                            temperatures=temperatures, noise=noise)
+                                            temperatures=temperatures, **self._noise_args(logits))
         x_cpu, transfer_cpu = x.cpu(), transfer.cpu()
         for i, seq in enumerate(seqs):
             seq.current_denoising_block = x_cpu[i]

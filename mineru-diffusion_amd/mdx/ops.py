@@ -261,12 +261,40 @@ def _logits2d(logits: torch.Tensor) -> torch.Tensor:
     return l2
 
 
+def _generator_args(seed, offset, offset_dev, row_ids, rows):
+    """(seed, offset, offset_dev pointer, row_ids pointer) of the in-kernel Gumbel generator."""
+    if offset_dev is not None:
+        assert offset_dev.dtype == torch.int64 and offset_dev.numel() == 1 and offset_dev.is_cuda
+    if row_ids is not None:
+        assert row_ids.dtype == torch.int64 and row_ids.numel() == rows and row_ids.is_contiguous() and row_ids.is_cuda
+    return (int(seed) & (2 ** 64 - 1), int(offset) & (2 ** 64 - 1),
+            None if offset_dev is None else offset_dev.data_ptr(), None if row_ids is None else row_ids.data_ptr())
+
+
+def gumbel_noise(rows: int, vocab: int, seed: int, offset: int = 0, device=None,
+                 offset_dev: torch.Tensor | None = None, row_ids: torch.Tensor | None = None) -> torch.Tensor:
+    """The [rows, vocab] fp32 noise tensor that `seed` / `offset` stand for in confidence_argmax and
+    unmask_step: passing it as `noise` gives the same result as passing the two integers."""
+    out = torch.empty((rows, vocab), dtype=torch.float32, device=device if device is not None else "cuda")
+    _need_gpu(out, offset_dev, row_ids)
+    rc = _lib.lib().mdx_gumbel_noise(out.data_ptr(), out.stride(0) if rows else vocab, rows, vocab,
+                                     *_generator_args(seed, offset, offset_dev, row_ids, rows), _stream(out))
+    check(rc, "gumbel_noise")
+    return out
+
+
 def confidence_argmax(logits: torch.Tensor, temperatures: torch.Tensor | None = None,
-                      noise: torch.Tensor | None = None):
-    """Sampler.prepare (nanovllm/layers/sampler.py:11-22) without its internal RNG:
+                      noise: torch.Tensor | None = None, seed: int | None = None, offset: int = 0,
+                      offset_dev: torch.Tensor | None = None, row_ids: torch.Tensor | None = None):
+    """Sampler.prepare (nanovllm/layers/sampler.py:11-22):
     logits [bs, S, V], temperatures [bs] or [bs, 1] fp32 -> (x0 int64 [bs, S], x0_p fp32 [bs, S]).
-    `noise` ([bs, S, V] fp32) is added to logits/T before the argmax; None = plain argmax."""
+    The Gumbel noise that the reference adds to logits/T before the argmax is either an explicit tensor
+    `noise` ([bs, S, V] fp32), or drawn inside the kernel from (`seed`, `offset`): a counter-based
+    generator, so the same integers give the same tokens (give every step another offset; `offset_dev`,
+    a one-element int64 device tensor, is added to it at run time; `row_ids` [rows] int64 names the
+    generator row of each logits row when rows were compacted).  Neither = plain argmax."""
     _need_gpu(logits, temperatures, noise)
+    assert noise is None or seed is None, "either a noise tensor or a seed"
     lead = logits.shape[:-1]
     l2 = _logits2d(logits)
     rows, vocab = l2.shape
@@ -286,8 +314,13 @@ def confidence_argmax(logits: torch.Tensor, temperatures: torch.Tensor | None = 
     L = _lib.lib()
     ws_bytes = L.mdx_confidence_argmax_workspace_bytes(rows, vocab)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=logits.device)
-    rc = L.mdx_confidence_argmax(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, rows_per_temp, n_ptr, n_stride,
-                                 x0.data_ptr(), x0_p.data_ptr(), rows, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    if seed is not None:
+        rc = L.mdx_confidence_argmax_gumbel(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, rows_per_temp,
+                                            *_generator_args(seed, offset, offset_dev, row_ids, rows),
+                                            x0.data_ptr(), x0_p.data_ptr(), rows, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    else:
+        rc = L.mdx_confidence_argmax(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, rows_per_temp, n_ptr, n_stride,
+                                     x0.data_ptr(), x0_p.data_ptr(), rows, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
     check(rc, "confidence_argmax")
     return x0.view(lead), x0_p.view(lead)
 
@@ -339,11 +372,14 @@ def select_transfer(x0: torch.Tensor, x0_p: torch.Tensor, tokens: torch.Tensor, 
 
 def unmask_step(logits: torch.Tensor, tokens: torch.Tensor, mask_token_id: int, threshold: float, k: int = 1,
                 temperatures: torch.Tensor | None = None, noise: torch.Tensor | None = None,
-                top_k: int = 0, top_p: float = 1.0):
+                top_k: int = 0, top_p: float = 1.0, seed: int | None = None, offset: int = 0,
+                offset_dev: torch.Tensor | None = None):
     """One whole unmask step on the device: logits [bs, S, V], tokens [bs, S] int64 (in place).
     Returns (x0, x0_p, transfer, count).  top_k / top_p (off by default, as in
-    modeling_mineru_diffusion.py:602,633-634) put filter_logits in front of the step."""
+    modeling_mineru_diffusion.py:602,633-634) put filter_logits in front of the step; `noise` or
+    (`seed`, `offset`, `offset_dev`) as for confidence_argmax."""
     _need_gpu(logits, tokens, temperatures, noise)
+    assert noise is None or seed is None, "either a noise tensor or a seed"
     if top_k > 0 or top_p < 1.0:
         logits = filter_logits(logits, top_k, top_p, temperatures)
     assert tokens.dtype == torch.int64 and tokens.is_contiguous()
@@ -368,9 +404,16 @@ def unmask_step(logits: torch.Tensor, tokens: torch.Tensor, mask_token_id: int, 
     L = _lib.lib()
     ws_bytes = L.mdx_confidence_argmax_workspace_bytes(rows, vocab)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
-    rc = L.mdx_unmask_step(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, n_ptr, n_stride,
-                           tokens.data_ptr(), int(mask_token_id), float(threshold), int(k),
-                           x0.data_ptr(), x0_p.data_ptr(), transfer.data_ptr(), count.data_ptr(),
-                           bs, S, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    if seed is not None:
+        rc = L.mdx_unmask_step_gumbel(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr,
+                                      *_generator_args(seed, offset, offset_dev, None, rows),
+                                      tokens.data_ptr(), int(mask_token_id), float(threshold), int(k),
+                                      x0.data_ptr(), x0_p.data_ptr(), transfer.data_ptr(), count.data_ptr(),
+                                      bs, S, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
+    else:
+        rc = L.mdx_unmask_step(l2.data_ptr(), l2.stride(0), _DTYPES[l2.dtype], t_ptr, n_ptr, n_stride,
+                               tokens.data_ptr(), int(mask_token_id), float(threshold), int(k),
+                               x0.data_ptr(), x0_p.data_ptr(), transfer.data_ptr(), count.data_ptr(),
+                               bs, S, vocab, ws.data_ptr(), ws_bytes, _stream(logits))
     check(rc, "unmask_step")
     return x0, x0_p, transfer.view(torch.bool), count

@@ -26,6 +26,10 @@ staircase_attn_varlen       block-b output independent of later blocks,
 paged_gather / paged attn   paged == contiguous, page permutation invariance
 store_kvcache               torch index_copy_, untouched slots, -1 skipped
 confidence_argmax           torch.softmax / torch.argmax, fp64 explicit sums
+philox4x32_10               the known-answer vectors of the Random123 distribution (zeros, all ones, digits of pi),
+                            distinct counters / keys give distinct outputs
+gumbel_noise                built on philox4x32_10; its uniforms lie in (0, 1) on a 2^-23 grid, mean / variance of
+                            the Gumbel law (Euler's constant, pi^2 / 6), Gumbel-max frequencies = softmax
 filter_logits               torch.topk / sort / cumsum / scatter formulation on tie-free rows, kept count == k,
                             kept mass exceeds p and stops exceeding it without its smallest element,
                             brute force over all cut-offs on 8 values, ties at the cut-off all kept
@@ -58,7 +62,7 @@ from .staircase import (  # noqa: F401
     attention_f64_explicit, staircase_attn_varlen, paged_gather, paged_block_attn,
 )
 from .kvstore import store_kvcache  # noqa: F401
-from .unmask import confidence_argmax, filter_logits, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
+from .unmask import confidence_argmax, filter_logits, philox4x32_10, gumbel_noise, select_transfer, unmask_step, num_transfer_tokens  # noqa: F401
 from .slots import slot_of, get_slots  # noqa: F401
 from .engine import dense_forward, expected_passes, block_prepare, masked_rows, block_advance  # noqa: F401
 from .fused import qk_norm_rope, rms_norm_ref, rope_ref, add_rms_norm, silu_and_mul  # noqa: F401

@@ -38,6 +38,46 @@ def confidence_argmax(logits: np.ndarray, temperatures=None, noise: np.ndarray |
     return x0, chosen / e.sum(axis=-1)
 
 
+_PHILOX_M0, _PHILOX_M1 = 0xD2511F53, 0xCD9E8D57
+_PHILOX_W0, _PHILOX_W1 = 0x9E3779B9, 0xBB67AE85
+
+
+def philox4x32_10(counter, key):
+    """Philox-4x32 with 10 rounds (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+    SC 2011; the generator of the Random123 library): counter = 4 arrays of uint32, key = 2 uint32 ->
+    4 arrays of uint32.  A round maps (c0, c1, c2, c3) to (hi(M1 c2) ^ c1 ^ k0, lo(M1 c2), hi(M0 c0) ^ c3 ^ k1,
+    lo(M0 c0)); the key is bumped by the Weyl constants between rounds."""
+    c = [np.asarray(x, dtype=np.uint64) & 0xFFFFFFFF for x in counter]
+    k0, k1 = int(key[0]) & 0xFFFFFFFF, int(key[1]) & 0xFFFFFFFF
+    for _ in range(10):
+        p0 = _PHILOX_M0 * c[0]
+        p1 = _PHILOX_M1 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k0, p1 & 0xFFFFFFFF, (p0 >> 32) ^ c[3] ^ k1, p0 & 0xFFFFFFFF]
+        k0 = (k0 + _PHILOX_W0) & 0xFFFFFFFF
+        k1 = (k1 + _PHILOX_W1) & 0xFFFFFFFF
+    return [x.astype(np.uint32) for x in c]
+
+
+def gumbel_noise(rows: int, vocab: int, seed: int, offset: int = 0, row_ids=None) -> np.ndarray:
+    """The noise that the library's in-kernel generator stands for, [rows, vocab] float64:
+    sampler.py:15-16 draws gumbel = -log(Exponential(1)); here element (row, column) takes output
+    column % 4 of Philox-4x32-10 with key = (seed low, seed high) and counter = (column // 4, row,
+    offset low, offset high), turns its 32 bits r into u = ((r >> 9) + 1/2) / 2^23 in (0, 1),
+    e = -ln u (a unit exponential) and returns -ln e."""
+    rid = np.arange(rows, dtype=np.uint64) if row_ids is None else np.asarray(row_ids, dtype=np.uint64)
+    groups = (vocab + 3) // 4
+    g = np.arange(groups, dtype=np.uint64)
+    c0 = np.broadcast_to(g[None, :], (rows, groups))
+    c1 = np.broadcast_to(rid[:, None], (rows, groups))
+    off = int(offset) & (2 ** 64 - 1)
+    c2 = np.full((rows, groups), off & 0xFFFFFFFF, dtype=np.uint64)
+    c3 = np.full((rows, groups), off >> 32, dtype=np.uint64)
+    out = philox4x32_10((c0, c1, c2, c3), (int(seed) & 0xFFFFFFFF, (int(seed) >> 32) & 0xFFFFFFFF))
+    bits = np.stack(out, axis=-1).reshape(rows, groups * 4)[:, :vocab]
+    u = ((bits >> 9).astype(np.float64) + 0.5) / 2.0 ** 23
+    return -np.log(-np.log(u))
+
+
 def filter_logits(logits: np.ndarray, top_k: int = 0, top_p: float = 1.0, temperatures=None) -> np.ndarray:
     """logits [rows, V] -> float64 copy with the filtered-out elements at -inf.
 
@@ -80,7 +120,9 @@ def select_transfer(conf: np.ndarray, masked: np.ndarray, threshold: float, k: i
 
     Defined here where the reference leaves it open: among equal confidences the
     LOWER position wins, and at most #masked positions are committed (the
-    reference's topk would otherwise return already-committed -inf positions).
+    reference's topk would otherwise return already-committed -inf positions);
+    a masked position whose confidence is -inf (no softmax ever gives that) is
+    never committed, so a caller can mark positions it has no confidence for.
     The engine variant (sampler.py:41-50: skip rows without masked positions,
     all of hi if any else top-1) is this rule with k = 1.
     """
@@ -93,12 +135,13 @@ def select_transfer(conf: np.ndarray, masked: np.ndarray, threshold: float, k: i
         if hi.sum() >= k:
             out[b] = hi
             continue
-        want = min(k, int(masked[b].sum()))
+        eligible = masked[b] & (c > -np.inf)
+        want = min(k, int(eligible.sum()))
         taken = np.zeros_like(hi)
         for _ in range(want):
             best = -1
             for p in range(c.shape[0]):
-                if masked[b, p] and not taken[p] and (best < 0 or c[p] > c[best]):
+                if eligible[p] and not taken[p] and (best < 0 or c[p] > c[best]):
                     best = p
             taken[best] = True
         out[b] = taken

@@ -223,21 +223,25 @@ def test_replay_ahead_changes_nothing(dev):
 
 def test_gumbel_noise_is_reproducible_per_seed(dev):
     """Sampler.prepare adds Gumbel noise to the scaled logits before the argmax (sampler.py:15-18);
-    here the noise comes from a seeded device generator: same seed, same tokens; another seed or no
-    noise, other tokens (temperature 1 on a random-weight model: the argmax is far from certain)."""
+    here the noise is drawn inside the unmask kernel as a function of (seed, sampling pass, row, column):
+    same seed, same tokens -- through the device loop with logits of the masked rows only, with logits of
+    all rows, and through the host-driven passes; another seed or no noise, other tokens (temperature 1
+    on a random-weight model: the argmax is far from certain)."""
     from mdx.engine import BlockDiffusionEngine, SamplingParams
     cfg, model = _tiny(dev)
     outs = {}
     for key, kw in (("a", dict(gumbel_seed=7)), ("b", dict(gumbel_seed=7)), ("c", dict(gumbel_seed=8)), ("plain", {}),
-                    ("full", dict(gumbel_seed=7, masked_rows_only=False))):
-        eng = BlockDiffusionEngine(model, num_pages=10, shuffle_pages_seed=3, decode_graphs=True, max_model_len=1024, **kw)
+                    ("full", dict(gumbel_seed=7, masked_rows_only=False)), ("host", dict(gumbel_seed=7, decode_graphs=False)),
+                    ("lockstep", dict(gumbel_seed=7, replay_ahead=False))):
+        kw = {"decode_graphs": True, **kw}
+        eng = BlockDiffusionEngine(model, num_pages=10, shuffle_pages_seed=3, max_model_len=1024, **kw)
         s = eng.add_request(list(range(5, 200)), SamplingParams(max_new_tokens=64, ignore_eos=True, transfer_count=4))
         eng.generate()
         outs[key] = s.completion_token_ids
         assert len(outs[key]) == 64 and cfg.mask_token_id not in outs[key]
     assert outs["a"] == outs["b"]
     assert outs["a"] != outs["c"] and outs["a"] != outs["plain"]
-    assert len(outs["full"]) == 64                          # the full-logits path draws noise of another shape: other tokens, same rules
+    assert outs["full"] == outs["a"] == outs["host"] == outs["lockstep"]   # the draw does not depend on how the pass is run
 
 
 @pytest.mark.parametrize("graphs", [False, True])

@@ -147,6 +147,28 @@ def test_unmask_fewer_masked_than_k_and_none(dev):
     assert etr.sum(-1).tolist() == [1, 2, 0]
 
 
+@pytest.mark.parametrize("S", [32, 100])
+def test_select_never_commits_a_position_without_a_confidence(dev, S):
+    """A masked position whose confidence is -inf (a caller's mark for "no fresh logits") stays masked and does
+    not use up one of the k places: wavefront kernel (S <= 64) and workgroup kernel."""
+    import mdx
+    g = torch.Generator().manual_seed(S)
+    bs = 5
+    conf = torch.rand(bs, S, generator=g)
+    conf[torch.rand(bs, S, generator=g) < 0.4] = float("-inf")
+    conf[4] = float("-inf")                                                       # a sequence with no confidence at all
+    x0 = torch.randint(0, 1000, (bs, S), generator=g)
+    tokens = torch.where(torch.rand(bs, S, generator=g) < 0.7, torch.tensor(MASK_ID), torch.randint(0, 1000, (bs, S), generator=g))
+    for thr, k in ((0.5, 3), (2.0, 6), (2.0, S)):
+        dtok = tokens.clone().to(dev)
+        tr, cnt = mdx.select_transfer(x0.to(dev), conf.to(dev), dtok, MASK_ID, thr, k)
+        torch.cuda.synchronize()
+        want = oracle.select_transfer(conf.numpy(), tokens.numpy() == MASK_ID, thr, k)
+        assert np.array_equal(tr.cpu().numpy(), want)
+        assert not (tr.cpu() & torch.isinf(conf)).any() and int(cnt[4]) == 0
+        assert np.array_equal(dtok.cpu().numpy(), np.where(want, x0.numpy(), tokens.numpy()))
+
+
 def test_unmask_block_lengths(dev):
     g = torch.Generator().manual_seed(8)
     for S in (1, 4, 33, 64, 128):

@@ -128,6 +128,10 @@ def test_select_strict_threshold_ties_and_engine_rule():
     assert oracle.select_transfer(conf, masked, 0.5, 1).tolist() == [[True, True, False, False]]
     # rows without masked positions commit nothing (sampler.py:42-43)
     assert not oracle.select_transfer(conf, np.zeros((1, 4), bool), 0.5, 1).any()
+    # a masked position without a confidence (-inf) is never committed, and does not use up one of the k places
+    gaps = np.array([[-np.inf, 0.2, -np.inf, 0.1]], np.float32)
+    assert oracle.select_transfer(gaps, masked, 0.5, 3).tolist() == [[False, True, False, True]]
+    assert not oracle.select_transfer(np.full((1, 4), -np.inf, np.float32), masked, 0.5, 2).any()
 
 
 def test_unmask_step_end_to_end_small():
@@ -209,3 +213,44 @@ def test_filter_brute_force_and_ties():
     y = np.array([[0.0, -np.inf, 1.0, -np.inf], [-np.inf] * 4])
     f = oracle.filter_logits(y, top_k=3, top_p=0.99)
     assert np.array_equal(np.isfinite(f), [[True, False, True, False], [False] * 4])
+
+
+# ---- the counter-based generator behind the in-kernel Gumbel noise ------------------------------
+
+def test_philox_known_answers():
+    """The three known-answer vectors that the Random123 distribution ships for philox4x32 with 10 rounds
+    (kat_vectors: counter words, key words -> output words)."""
+    kat = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+           ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+           ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0), (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kat:
+        got = oracle.philox4x32_10([np.array([w]) for w in ctr], key)
+        assert tuple(int(g[0]) for g in got) == want
+    # vectorised over counters = one at a time; neighbouring counters and keys give unrelated words
+    c = [np.arange(5), np.zeros(5), np.full(5, 7), np.zeros(5)]
+    many = oracle.philox4x32_10(c, (1, 2))
+    for i in range(5):
+        one = oracle.philox4x32_10([np.array([x[i]]) for x in c], (1, 2))
+        assert all(int(one[j][0]) == int(many[j][i]) for j in range(4))
+    assert len({int(w) for out in many for w in out}) == 20
+    assert int(oracle.philox4x32_10(c, (1, 3))[0][0]) != int(many[0][0])
+
+
+def test_gumbel_noise_law_and_coordinates():
+    g = oracle.gumbel_noise(64, 4099, seed=11, offset=5)
+    assert g.shape == (64, 4099) and np.isfinite(g).all()
+    assert -2.82 < g.min() and g.max() < 16.65                     # -ln(-ln u) for u on the 2^-23 grid inside (0, 1)
+    assert abs(g.mean() - 0.5772156649) < 0.01 and abs(g.var() - np.pi ** 2 / 6) < 0.03
+    # a pure function of (seed, offset, row, column): rows and offsets are separate streams, row_ids relabel rows
+    assert np.array_equal(oracle.gumbel_noise(3, 50, 11, 5), g[:3, :50])
+    assert not np.array_equal(oracle.gumbel_noise(3, 50, 11, 6), g[:3, :50])
+    assert not np.array_equal(oracle.gumbel_noise(3, 50, 12, 5), g[:3, :50])
+    assert np.array_equal(oracle.gumbel_noise(2, 50, 11, 5, row_ids=[40, 7]), g[[40, 7], :50])
+    big = oracle.gumbel_noise(1, 8, seed=2 ** 40 + 3, offset=2 ** 35 + 1)            # high words of seed and offset matter
+    assert not np.array_equal(big, oracle.gumbel_noise(1, 8, seed=3, offset=1))
+    # Gumbel-max: argmax(l + g) is a draw from softmax(l)
+    l = np.array([0.0, 1.0, 2.0, -1.0, 0.5])
+    draws = (l[None, :] + oracle.gumbel_noise(40000, 5, seed=1)).argmax(1)
+    freq = np.bincount(draws, minlength=5) / 40000
+    want = np.exp(l) / np.exp(l).sum()
+    assert np.abs(freq - want).max() < 0.01
