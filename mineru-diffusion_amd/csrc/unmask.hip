@@ -121,9 +121,8 @@ template <> struct Elem<float> {
     static __device__ __forceinline__ float one(const float* p) { return *p; }
 };
 
-// One element through the slow path (row head/tail, and every element when a
-// noise tensor is given).  With noise, l = x / T is a true fp32 division so the
-// noisy argmax matches an fp32 host computation bit for bit.
+// One element through the slow path (row head/tail).  With noise, l = x / T is a
+// true fp32 division so the noisy argmax matches an fp32 host computation bit for bit.
 template <bool NOISE>
 __device__ __forceinline__ void visit(Partial& p, float x, int index, float c, float T, float g) {
     if (x > p.m) {
@@ -312,33 +311,46 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
             for (int64_t e = tid; e < lead; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
             for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<false>(p, Elem<T>::one(rp + e), (int)e, c, T_, 0.f);
         }
-    } else if (NOISE == 1) {
-        // Noise path: 4 more bytes per element and a true division; element-wise.
-        const int64_t ebeg = (split == 0) ? 0 : lead + cbeg * EPC;
-        const int64_t eend = (split == nsplit - 1) ? vocab : lead + cend * EPC;
-        for (int64_t e = ebeg + tid; e < eend; e += kThreads)
-            visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, np[e]);
     } else {
-        // Noise from the generator.  The softmax runs over 16-byte chunks as without noise; the noisy argmax is
-        // the arithmetic of the tensor path element by element (l = x / T by a true division, v = l + g, the
-        // larger v or at equal v the lower index wins), so both paths draw the same tokens.  A chunk whose first
-        // column is a multiple of 4 (every row that starts on a 16-byte boundary) takes whole generator
-        // outputs, EPC / 4 of them; otherwise every element asks for its own.
-        const RowNoise rn = row_noise(N, row);
+        // With noise.  The softmax runs over 16-byte chunks as without noise; the noisy argmax is element by
+        // element: l = x / T by a true division (skipped, not approximated, when T = 1: x / 1 == x), v = l + g, the
+        // larger v or at equal v the lower index wins -- the arithmetic of an fp32 host computation, bit for bit.
+        // The noise g of an element is read from the tensor (mode 1; 16-byte loads when the row's noise lines up
+        // with its chunks) or drawn from the generator (mode 2: a chunk whose first column is a multiple of 4 --
+        // every row that starts on a 16-byte boundary -- takes whole generator outputs, EPC / 4 of them; otherwise
+        // every element asks for its own), so both modes draw the same tokens from the same noise.
+        const RowNoise rn = NOISE == 2 ? row_noise(N, row) : RowNoise{0, 0, 0, 0, 0};
         const bool whole_groups = (lead & 3) == 0;
-        const bool unit_T = T_ == 1.0f;                 // x / 1 == x: the division is skipped, not approximated
+        const bool noise_lines_up = NOISE == 1 && (reinterpret_cast<uintptr_t>(np + lead) & 15) == 0;
+        const bool unit_T = T_ == 1.0f;
         float best = kNegBig, best_x = 0.f;
         int best_idx = kNoIndex;
         auto offer = [&](float x, int index, float g) {
             const float v = (unit_T ? x : x / T_) + g;
             if (v > best || (v == best && index < best_idx)) { best = v; best_x = x; best_idx = index; }
         };
+        auto noise_at = [&](int64_t e) { return NOISE == 1 ? np[e] : rn.at((int)e); };
         for (int64_t ch = cbeg + tid; ch < cend; ch += kThreads) {
             float x[EPC];
             Elem<T>::unpack(__builtin_nontemporal_load(cp + ch), x);
             take_values(x, ch);
             const int c0 = (int)(lead + ch * EPC);
-            if (whole_groups) {
+            if (NOISE == 1) {
+                float g[EPC];
+                if (noise_lines_up) {
+#pragma unroll
+                    for (int q = 0; q < EPC / 4; ++q) {
+                        const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(np + c0) + q);
+                        g[4 * q + 0] = __uint_as_float(w.x); g[4 * q + 1] = __uint_as_float(w.y);
+                        g[4 * q + 2] = __uint_as_float(w.z); g[4 * q + 3] = __uint_as_float(w.w);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < EPC; ++i) g[i] = np[c0 + i];
+                }
+#pragma unroll
+                for (int i = 0; i < EPC; ++i) offer(x[i], c0 + i, g[i]);
+            } else if (whole_groups) {
 #pragma unroll
                 for (int q = 0; q < EPC / 4; ++q) {
                     const U4 r = rn.group((uint32_t)(c0 >> 2) + q);
@@ -355,8 +367,8 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
         lane_softmax_done();
         p.pick = best; p.pick_x = best_x; p.pick_idx = best_idx;
         if (split == 0) {
-            for (int64_t e = tid; e < lead; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, rn.at((int)e));
-            for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, rn.at((int)e));
+            for (int64_t e = tid; e < lead; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, noise_at(e));
+            for (int64_t e = tail0 + tid; e < vocab; e += kThreads) visit<true>(p, Elem<T>::one(rp + e), (int)e, c, T_, noise_at(e));
         }
     }
 
