@@ -568,7 +568,7 @@ def main():
                 assert rc == 0
             fl_ms, fl_min = time_kernel(logit_filter, 2, max(3, K // 4), graph=True)
             result_ops["filter_logits"] = op_entry(fl_ms, fl_min, "hbm", 2 * c4["bytes"], 1e6, PEAK_HBM_GBS, "GB/s",
-                                                   dict(top_k=50, top_p=0.9, note="off by default in the reference; reads each row four to five times"))
+                                                   dict(top_k=50, top_p=0.9, note="off by default in the reference; with both filters on a row is read six times (five counting passes and the writing pass)"))
             del flt_out
         del c4
         torch.cuda.empty_cache()
