@@ -110,6 +110,32 @@ def test_sampler_forward_over_several_steps_unmasks_the_block(dev):
     assert total == 2 * S and not (cur == MASK_ID).any()        # 4 per step x 8 steps
 
 
+def test_sampler_with_a_seed_samples_like_the_reference_prepare(dev):
+    """Sampler(seed=) draws the Gumbel noise of sampler.py:15-16 inside the kernel: the Sequences change exactly as the
+    oracle's step on the oracle's restatement of that noise says, every call takes the next offset, and the same
+    seed replays the same calls."""
+    import mdx
+    logits, tokens, temps = _sampler_case(seed=9)
+    bs, S, V = logits.shape
+    l64 = logits.to(torch.float64).numpy()
+    for attempt in range(2):
+        sampler = mdx.Sampler(k=1, seed=4242)
+        cur = tokens.numpy().copy()
+        seqs = _fake_seqs(tokens.clone(), 0.9, [0] * bs)
+        for call in range(3):
+            noise = oracle.gumbel_noise(bs * S, V, 4242, offset=call).reshape(bs, S, V)
+            ex0, ep, etr, etok = oracle.unmask_step(l64, cur, MASK_ID, 0.9, 1, temperatures=temps.numpy().reshape(-1), noise=noise)
+            n = sampler.forward(logits.to(dev), temps.to(dev), seqs)
+            assert n == int(etr.sum())
+            for i, s in enumerate(seqs):
+                assert np.array_equal(s.current_denoising_block.numpy(), etok[i]), f"call {call}, sequence {i}"
+            cur = etok
+        assert sampler.calls == 3
+    x0_plain, _ = mdx.Sampler().prepare(logits.to(dev), temps.to(dev))
+    x0_noisy, _ = mdx.Sampler(seed=4242).prepare(logits.to(dev), temps.to(dev))
+    assert not torch.equal(x0_plain, x0_noisy)
+
+
 def test_sampler_prepare_is_the_confidence_pass(dev):
     import mdx
     logits, _, temps = _sampler_case(seed=8, bs=3)
