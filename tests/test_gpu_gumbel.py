@@ -15,14 +15,18 @@ def _f64(t):
     return t.detach().cpu().to(torch.float64).numpy()
 
 
-@pytest.mark.parametrize("rows,vocab,seed,offset", [(3, 1, 0, 0), (5, 7, 1, 0), (4, 4096, 123456789, 17), (2, 151936, 2 ** 40 + 3, 2 ** 35 + 1)])
+@pytest.mark.parametrize("rows,vocab,seed,offset", [(3, 1, 0, 0), (5, 7, 1, 0), (4, 4096, 123456789, 17), (40, 151936, 2 ** 40 + 3, 2 ** 35 + 1)])
 def test_noise_tensor_matches_the_oracle_generator(dev, rows, vocab, seed, offset):
     import mdx
     got = mdx.gumbel_noise(rows, vocab, seed, offset, device=dev)
     torch.cuda.synchronize()
     want = oracle.gumbel_noise(rows, vocab, seed, offset)
-    # same random bits (a wrong word would be off by O(1)); fp32 logarithms against fp64 ones
-    np.testing.assert_allclose(_f64(got), want, rtol=2e-6, atol=2e-6)
+    # same random bits (a wrong word would be off by O(1)); fp32 logarithms against fp64 ones.  The largest case
+    # holds 6 million draws: its largest noise values (above 14, from u within 1e-6 of 1, the draws that decide an
+    # argmax) are as accurate as the rest.
+    np.testing.assert_allclose(_f64(got), want, rtol=0, atol=3e-6)
+    if rows * vocab > 10 ** 6:
+        assert want.max() > 14
 
 
 def test_noise_row_ids_and_device_offset(dev):
@@ -31,23 +35,9 @@ def test_noise_row_ids_and_device_offset(dev):
     bump = torch.tensor([5], dtype=torch.int64, device=dev)
     got = mdx.gumbel_noise(3, 1001, 77, 20, device=dev, offset_dev=bump, row_ids=ids)
     torch.cuda.synchronize()
-    np.testing.assert_allclose(_f64(got), oracle.gumbel_noise(3, 1001, 77, 25, row_ids=[9, 0, 4]), rtol=2e-6, atol=2e-6)
+    np.testing.assert_allclose(_f64(got), oracle.gumbel_noise(3, 1001, 77, 25, row_ids=[9, 0, 4]), rtol=0, atol=3e-6)
     full = mdx.gumbel_noise(10, 1001, 77, 25, device=dev)
     assert torch.equal(got, full[ids])                      # the same bits as the uncompacted layout
-
-
-def test_largest_draws_keep_their_accuracy(dev):
-    """u next to 1 gives the largest noise, the draws that decide an argmax: -ln u is taken from a series
-    there.  Checked on all 2^23 values of u through the same arithmetic as the kernel's, in torch fp32 on the GPU,
-    which this test states again (so it pins the formula, not the kernel)."""
-    k = torch.arange(2 ** 23, device=dev, dtype=torch.float32)
-    u64 = (k.double() + 0.5) / 2 ** 23
-    want = -torch.log(-torch.log(u64))
-    w = (8388607.5 - k) * 2.0 ** -23
-    series = w * (1 + w * (0.5 + w * (0.33333334 + w * 0.25)))
-    e = torch.where(w < 0.015625, series, -torch.log(((k + 0.5) * 2.0 ** -23)))
-    got = -torch.log(e)
-    assert (got.double() - want).abs().max().item() < 4e-6
 
 
 def _case(dev, dtype, bs, S, V, seed, offset, temps=None, stride=None):
