@@ -273,7 +273,7 @@ int mdx_gumbel_noise(float* noise, int64_t noise_row_stride, int64_t rows, int64
  * cut-off value set to -inf, to be passed on to mdx_confidence_argmax / mdx_unmask_step (whose noise
  * input then samples from the filtered distribution as torch.multinomial does at :613).
  *
- * logits, out: [rows, vocab], MDX_BF16 or MDX_F16 (the cut-off is found by counting over the 65 536
+ * logits, out: [rows, vocab <= 2^23], MDX_BF16 or MDX_F16 (the cut-off is found by counting over the 65 536
  * values a 16-bit element can take; MDX_F32 is refused), row strides in elements; out may be logits
  * itself.  top_k = 0 (or >= vocab) switches the top-k filter off, top_p >= 1 the top-p filter.
  * top-k keeps the elements >= the k-th largest value (equal values are all kept, as in the reference);

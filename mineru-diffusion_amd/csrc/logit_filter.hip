@@ -247,8 +247,9 @@ extern "C" int mdx_filter_logits(const void* logits, int64_t row_stride, int32_t
     MDX_REQUIRE(vocab > 0, MDX_EINVAL, "filter_logits: empty vocabulary");
     MDX_REQUIRE(logits && out, MDX_EINVAL, "filter_logits: null pointer");
     MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "filter_logits: dtype %d (16-bit logits only)", dtype);
-    MDX_REQUIRE(vocab < (int64_t)0x7fffffff && rows < (int64_t)0x7fffffff, MDX_EUNSUPPORTED,
-                "filter_logits: rows %lld or vocab %lld out of range", (long long)rows, (long long)vocab);
+    // a bin's mass is a 64-bit sum of terms of up to 2^40 each: exact for rows of up to 2^23 elements
+    MDX_REQUIRE(vocab <= (int64_t)1 << 23 && rows < (int64_t)0x7fffffff, MDX_EUNSUPPORTED,
+                "filter_logits: rows %lld or vocab %lld out of range (vocab at most 8388608)", (long long)rows, (long long)vocab);
     MDX_REQUIRE(row_stride >= vocab && out_row_stride >= vocab, MDX_EUNSUPPORTED, "filter_logits: row stride smaller than the vocabulary");
     MDX_REQUIRE(!temperatures || rows_per_temp > 0, MDX_EINVAL, "filter_logits: rows_per_temp must be positive");
     MDX_REQUIRE((reinterpret_cast<uintptr_t>(logits) % 2) == 0 && (reinterpret_cast<uintptr_t>(out) % 2) == 0,
