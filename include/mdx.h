@@ -214,7 +214,9 @@ int mdx_confidence_argmax(const void* logits, int64_t row_stride, int32_t dtype,
  * confident masked positions (ties: lower position first; a position whose
  * x0_p is -inf is never committed, which lets a caller mark rows it has no
  * fresh confidence for).  k = 1 gives the
- * engine's rule (sampler.py:41-50), k = block/steps the HF rule.  Writes
+ * engine's rule (sampler.py:41-50), k = block/steps the HF rule (k = 0, which
+ * its schedule reaches when a block has fewer positions than steps, commits
+ * the positions above the threshold and no others).  Writes
  * transfer[b,p] (uint8 0/1), tokens[b,p] = x0[b,p] where committed (in place),
  * and count[b] = number committed (int32).
  */

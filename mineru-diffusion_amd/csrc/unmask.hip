@@ -708,7 +708,7 @@ extern "C" int mdx_select_transfer(const int64_t* x0, const float* x0_p, int64_t
     if (bs == 0 || block_len == 0) return MDX_OK;
     MDX_REQUIRE(x0 && x0_p && tokens && transfer && count, MDX_EINVAL, "select_transfer: null pointer");
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "select_transfer: block_len %d > %d", block_len, kMaxBlockLen);
-    MDX_REQUIRE(k >= 1, MDX_EINVAL, "select_transfer: k %d < 1", k);
+    MDX_REQUIRE(k >= 0, MDX_EINVAL, "select_transfer: k %d < 0", k);
     return launch_select(const_cast<int64_t*>(x0), const_cast<float*>(x0_p), tokens, nullptr, 1, nullptr, mask_token_id, threshold, k,
                          transfer, count, bs, block_len, stream);
 }
@@ -723,7 +723,7 @@ int unmask_step_impl(const void* logits, int64_t row_stride, int32_t dtype,
                      void* workspace, int64_t workspace_bytes, hipStream_t stream)
 {
     MDX_REQUIRE(bs >= 0 && block_len >= 0, MDX_EINVAL, "unmask_step: negative size");
-    MDX_REQUIRE(k >= 1, MDX_EINVAL, "unmask_step: k %d < 1", k);
+    MDX_REQUIRE(k >= 0, MDX_EINVAL, "unmask_step: k %d < 0", k);
     MDX_REQUIRE(block_len <= kMaxBlockLen, MDX_EUNSUPPORTED, "unmask_step: block_len %d > %d", block_len, kMaxBlockLen);
     if (bs == 0 || block_len == 0) return MDX_OK;
     MDX_REQUIRE(tokens && transfer && count, MDX_EINVAL, "unmask_step: null pointer");

@@ -353,6 +353,14 @@ def filter_logits(logits: torch.Tensor, top_k: int = 0, top_p: float = 1.0,
     return out
 
 
+def num_transfer_tokens(block_length: int, steps: int) -> list[int]:
+    """get_num_transfer_tokens (modeling_mineru_diffusion.py:617-623): how many positions each denoising step of a
+    block commits at least -- block_length split over the steps, the remainder given to the first steps.  The k of
+    unmask_step / select_transfer for step i is entry min(i, steps - 1) (modeling_mineru_diffusion.py:712)."""
+    base, rem = divmod(int(block_length), int(steps))
+    return [base + (1 if i < rem else 0) for i in range(int(steps))]
+
+
 def select_transfer(x0: torch.Tensor, x0_p: torch.Tensor, tokens: torch.Tensor, mask_token_id: int,
                     threshold: float, k: int = 1):
     """Device form of the selection loop (sampler.py:32-54, modeling_mineru_diffusion.py:518-532).

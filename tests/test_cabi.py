@@ -71,7 +71,7 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     assert pa(sq=33) == -2
     assert pa(page=100) == -2
     assert pa() == -3 and b"workspace" in L.mdx_last_error()
-    assert L.mdx_select_transfer(one, one, one, 7, 0.9, 0, one, one, 2, 32, null) == -1       # k < 1
+    assert L.mdx_select_transfer(one, one, one, 7, 0.9, -1, one, one, 2, 32, null) == -1      # k < 0
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 1, one, one, 2, 2000, null) == -2      # block too long
     assert L.mdx_confidence_argmax(one, 10, 0, null, 1, null, 0, one, one, 4, 20, null, 0, null) == -2   # stride < vocab
     fl = lambda **kw: L.mdx_filter_logits(one, kw.get("stride", 100), kw.get("dtype", 0), null, 1,           # noqa: E731

@@ -227,3 +227,15 @@ def test_oracle_block_advance_stop_token_and_idle_lanes():
     assert appended[2] is None and appended[0][0].tolist() == list(range(10, 42))
     assert (t[0] == MASK).all() and (t[2] == tokens[2]).all() and step.tolist() == [5, 5, 4]
     assert status[1] == (1, 37, S, 0)
+
+
+def test_transfer_schedule_helper_matches_the_oracle():
+    """mdx.num_transfer_tokens is host arithmetic (modeling_mineru_diffusion.py:617-623): same lists as the oracle's,
+    which sum to the block length, differ by at most one and may hold zeros when a block is shorter than its steps."""
+    import mdx
+    for block, steps in ((32, 8), (32, 32), (10, 4), (32, 5), (3, 8), (1, 1)):
+        got = mdx.num_transfer_tokens(block, steps)
+        assert got == oracle.num_transfer_tokens(block, steps)
+        assert sum(got) == block and max(got) - min(got) <= 1 and got == sorted(got, reverse=True)
+    assert mdx.num_transfer_tokens(3, 8) == [1, 1, 1, 0, 0, 0, 0, 0]
+

@@ -169,6 +169,24 @@ def test_select_never_commits_a_position_without_a_confidence(dev, S):
         assert np.array_equal(dtok.cpu().numpy(), np.where(want, x0.numpy(), tokens.numpy()))
 
 
+def test_k_zero_commits_the_positions_above_the_threshold_only(dev):
+    """The HF schedule gives k = 0 to the late steps of a block with fewer positions than steps: hi.sum() >= 0 always
+    holds, so exactly the positions above the threshold are committed (modeling_mineru_diffusion.py:526-529)."""
+    import mdx
+    g = torch.Generator().manual_seed(12)
+    conf = torch.rand(4, 32, generator=g)
+    x0 = torch.randint(0, 1000, (4, 32), generator=g)
+    tokens = torch.where(torch.rand(4, 32, generator=g) < 0.6, torch.tensor(MASK_ID), torch.randint(0, 1000, (4, 32), generator=g))
+    dtok = tokens.clone().to(dev)
+    tr, cnt = mdx.select_transfer(x0.to(dev), conf.to(dev), dtok, MASK_ID, 0.7, 0)
+    torch.cuda.synchronize()
+    want = oracle.select_transfer(conf.numpy(), tokens.numpy() == MASK_ID, 0.7, 0)
+    assert np.array_equal(want, (tokens.numpy() == MASK_ID) & (conf.numpy() > 0.7))
+    assert np.array_equal(tr.cpu().numpy(), want) and cnt.cpu().tolist() == want.sum(1).tolist()
+    tr2, cnt2 = mdx.select_transfer(x0.to(dev), conf.to(dev), tokens.clone().to(dev), MASK_ID, 2.0, 0)
+    assert not tr2.any() and int(cnt2.sum()) == 0
+
+
 def test_unmask_block_lengths(dev):
     g = torch.Generator().manual_seed(8)
     for S in (1, 4, 33, 64, 128):
