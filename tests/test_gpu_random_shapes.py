@@ -82,3 +82,53 @@ def test_paged_random_shapes(dev):
         assert err < TOL, f"case {case}: max-abs {err}"
         assert torch.equal(one, two), f"case {case}: one launch differs from two"
         assert own.abs().sum().item() == 0
+
+
+def test_filter_and_seeded_sampling_random_shapes(dev):
+    """Random vocabulary sizes, row counts, alignments (rows that start off a 16-byte boundary), dtypes, temperatures
+    and filter settings: the filtered logits against the oracle's (rows whose top-p cut-off hinges on rounding aside),
+    and the step with noise drawn in the kernel against the step fed the same noise as a tensor (tokens bit for bit)."""
+    import mdx
+    rng = np.random.default_rng(777)
+    checked = 0
+    for case in range(20):
+        V = int(rng.choice([3, 17, 100, 1000, 4097, 30000, 151936]))
+        bs, S = int(rng.integers(1, 5)), int(rng.choice([1, 4, 32]))
+        rows = bs * S
+        dtype = torch.bfloat16 if case % 3 else torch.float16
+        pad = int(rng.integers(0, 8))                                   # row stride V + pad: most rows unaligned
+        g = torch.Generator().manual_seed(5000 + case)
+        buf = (torch.randn(rows, V + pad, generator=g) * float(rng.uniform(0.5, 4.0))).to(dtype)
+        logits = buf[:, :V]
+        temps = torch.tensor(rng.uniform(0.5, 2.0, bs), dtype=torch.float32)
+        k = int(rng.choice([0, 0, 1, 5, 50])) if V > 60 else int(rng.choice([0, 1, 2]))
+        p = float(rng.choice([1.0, 0.95, 0.7, 0.3]))
+        seed, offset = int(rng.integers(0, 2 ** 40)), int(rng.integers(0, 2 ** 34))
+        print(f"case {case}: V {V} bs {bs} S {S} {dtype} pad {pad} top_k {k} top_p {p}", flush=True)
+        d = buf.to(dev)[:, :V]
+        f = mdx.filter_logits(d, top_k=k, top_p=p, temperatures=temps.to(dev))
+        torch.cuda.synchronize()
+        x = logits.to(torch.float64).numpy()
+        T = np.repeat(temps.numpy().astype(np.float64), S)
+        want = oracle.filter_logits(x, top_k=k, top_p=p, temperatures=T)
+        got = f.to(torch.float64).cpu().numpy()
+        for r in range(rows):
+            if not np.array_equal(got[r], want[r]):                     # allowed only where a cumulative probability touches p
+                kept = x[r][np.isfinite(oracle.filter_logits(x[r:r + 1], top_k=k)[0])] / T[r]
+                vals, counts = np.unique(kept, return_counts=True)
+                mass = counts * np.exp(vals - vals[-1])
+                cum = np.cumsum(mass[::-1]) / mass.sum()
+                assert p < 1.0 and np.abs(cum - p).min() <= 2e-5, f"case {case} row {r}: kept set differs away from a rounding boundary"
+            else:
+                checked += 1
+        tokens = torch.where(torch.rand(bs, S, generator=g) < 0.7, torch.tensor(V + 5), torch.randint(0, V, (bs, S), generator=g))
+        t1, t2 = tokens.clone().to(dev), tokens.clone().to(dev)
+        a = mdx.unmask_step(f.view(bs, S, V), t1, V + 5, 0.4, 2, temps.to(dev), seed=seed, offset=offset)
+        noise = mdx.gumbel_noise(rows, V, seed, offset, device=dev).view(bs, S, V)
+        b = mdx.unmask_step(f.view(bs, S, V), t2, V + 5, 0.4, 2, temps.to(dev), noise=noise)
+        torch.cuda.synchronize()
+        assert torch.equal(a[0], b[0]) and torch.equal(a[2], b[2]) and torch.equal(t1, t2)
+        torch.testing.assert_close(a[1], b[1], rtol=3e-6, atol=0)
+        kept_mask = torch.isfinite(f.float()).view(bs, S, V)
+        assert bool(kept_mask.gather(-1, a[0].unsqueeze(-1)).all())      # a drawn token is always one that survived the filter
+    assert checked > 100
