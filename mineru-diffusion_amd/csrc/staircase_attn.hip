@@ -365,8 +365,12 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                                         : (int64_t)P.n_row_groups * batch;
     // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
     const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
-    // (the hand-scheduled pair kernel exists for bf16; fp16 runs the one-head kernel)
-    const bool pairs = dtype == MDX_BF16 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
+    // (the hand-scheduled pair kernel exists for bf16; fp16 runs the one-head kernel).  Sequences of a few hundred
+    // tokens are left to the one-head kernel as well: a pair workgroup owns a whole CU and its fixed cost (set-up,
+    // prologue, epilogue: 10 us) is then most of its time, while two one-head workgroups share a CU and hide each
+    // other's (64 x 600 tokens: 0.237 against 0.259 ms, 16 x 300: 0.028 against 0.035; equal at 1100 tokens, and
+    // from there on the pair kernel wins: 1.3 x at 8 x 4096).
+    const bool pairs = dtype == MDX_BF16 && max_l > 640 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");

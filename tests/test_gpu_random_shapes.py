@@ -39,6 +39,11 @@ def test_prefill_random_shapes(dev):
         ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
         err = (o.float().cpu() - ref).abs().max().item()
         assert err < TOL, f"case {case}: max-abs {err} (heads {hq}/{hkv}, S {S}, lens {lens})"
+        # a looser (still valid) length bound changes the launch grid and, for short batches, the kernel that runs
+        o2 = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S, max_seqlen=max(1024, max(lens)))
+        torch.cuda.synchronize()
+        err2 = (o2.float().cpu() - ref).abs().max().item()
+        assert err2 < TOL, f"case {case}: max-abs {err2} with a bound of {max(1024, max(lens))}"
 
 
 def test_paged_random_shapes(dev):
