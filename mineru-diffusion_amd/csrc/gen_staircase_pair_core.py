@@ -459,11 +459,31 @@ def select(cb):
     return [f".Ltop_{cb}_%=:",
             f"s_cmp_ge_i32 {S_T}, %[nt]",
             "s_cbranch_scc1 .Lend_%=",
+            f"s_cmp_ge_i32 {S_KEY0}, %[whx]",
+            "s_cbranch_scc1 .Lidle_%=",
             f"s_cmp_lt_i32 {S_KEY0}, %[pad]",
             f"s_cbranch_scc1 .Lmasked_{cb}_%=",
             f"s_add_i32 {S_TMP}, {S_KEY0}, 64",
             f"s_cmp_gt_i32 {S_TMP}, %[whm]",
             f"s_cbranch_scc1 .Lmasked_{cb}_%="]
+
+
+def idle_loop():
+    """Iterations whose tile lies wholly beyond the last key that any query of this wavefront may see (the other
+    wavefronts of the workgroup own later rows and still need the tile): nothing to compute -- every probability
+    would be zero -- but the wavefront keeps loading its quarter of every tile and meets the others at the barrier.
+    Entered from the top of an iteration, left only through the end of the loop."""
+    out = [".Lidle_%=:",
+           f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]
+    for first, last in dma_ops(S_R4):
+        out += first + ["s_nop 0"] + last
+    out += load_offset_ops()
+    out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_R3}",
+            f"s_mov_b32 {S_R3}, {S_R4}", f"s_mov_b32 {S_R4}, {S_TMP}",
+            f"s_add_i32 {S_T}, {S_T}, 1",
+            f"s_cmp_ge_i32 {S_T}, %[nt]",
+            "s_cbranch_scc0 .Lidle_%="]
+    return out
 
 
 def epilogue():
@@ -493,6 +513,7 @@ def program():
     out += select(0) + body(0, False) + select(1) + body(1, False) + ["s_branch .Ltop_0_%="]
     out += [".Lmasked_0_%=:"] + body(0, True) + ["s_branch .Ltop_1_%="]
     out += [".Lmasked_1_%=:"] + body(1, True) + ["s_branch .Ltop_0_%="]
+    out += idle_loop()
     out += epilogue()
     return out
 
@@ -514,7 +535,7 @@ struct PairCoreArgs {
     const void* kb; const void* vb;  // K / V of this KV head, at the (virtual) row of padded key 0
     unsigned krb, vrb;               // bytes between consecutive K / V rows
     unsigned wrow;                   // LDS byte address of the first row this wavefront loads in slot 0
-    int pad, lpm1, nt, whm;          // first valid padded key, last valid padded key, key tiles, first limit of this wavefront
+    int pad, lpm1, nt, whm, whx;     // first valid padded key, last valid padded key, key tiles, first and last key limit of this wavefront
 };
 
 __device__ __forceinline__ void staircase_pair_core(const PairCoreArgs& A, const bf16x8 (&q)[2][8])
@@ -535,7 +556,7 @@ def main():
         : [ka] "v"(A.ka), [val] "v"(A.val), [vah] "v"(A.vah), [jpl] "v"(A.jpl), [ch] "v"(A.ch),
           [mrel] "v"(A.mrel), [mlim] "v"(A.mlim), [o0] "v"(A.o0), [o1] "v"(A.o1), [ok] "v"(A.ok),
           [kb] "s"(A.kb), [vb] "s"(A.vb), [krb] "s"(A.krb), [vrb] "s"(A.vrb), [wrow] "s"(A.wrow),
-          [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm),
+          [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm), [whx] "s"(A.whx),
           {qops}
         : "memory", "vcc", "scc", "m0", {sclob},
           {vclob},

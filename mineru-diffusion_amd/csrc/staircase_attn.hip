@@ -221,8 +221,8 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 // needs 1 KB of LDS reads per MFMA and is bound by that).  512 registers per wavefront, one
 // workgroup per CU; the key loop is the hand-scheduled asm of staircase_pair_core.inc, in which the
 // softmax arithmetic of one tile is issued in the shadow of the next tile's QK MFMAs.  All four
-// wavefronts of a workgroup walk the same number of key tiles; tiles beyond a wavefront's own
-// limit are fully masked.
+// wavefronts of a workgroup walk the same number of key tiles (they share the tiles' loads and a
+// barrier per tile); for tiles beyond a wavefront's own last limit it only loads and waits.
 #include "staircase_pair_core.inc"
 
 constexpr int kPairSlots = 5;                     // LDS slots of one K tile + one V tile, 256-byte rows
@@ -311,6 +311,7 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.lpm1 = uniform(Lp - 1);
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
+    A.whx = uniform(row_w0 < Lp ? limit_of(min(row_w0 + 31, Lp - 1)) : 0);   // tiles from here on hold nothing this wavefront may see
     staircase_pair_core(A, q);
 }
 
