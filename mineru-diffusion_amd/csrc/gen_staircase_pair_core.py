@@ -454,6 +454,52 @@ def body(cb, masked):
     return out
 
 
+def body_last(cb):
+    """The iteration of the last tile that holds keys this wavefront may see: softmax and PV of tile t as in the
+    masked body, but no QK of tile t+1 (every one of its probabilities would be zero: the half of an ordinary
+    iteration's matrix work that the wavefront's first hidden tile used to cost).  The K fragment reads that the
+    previous iteration issued ahead are left to land unused.  Leaves into the idle loop."""
+    uid = f"{cb}L"
+    out = []
+    items = [None] * 16 + pv_items(cb)
+    plan = softmax_plan(cb, True)
+    tail = load_offset_ops()
+    per = -(-len(tail) // 6)
+    for i in range(6):
+        plan[26 + i] += tail[per * i:per * (i + 1)]
+    dma = dma_ops(S_R4)
+    rg = Ring()
+    rg.issued = RING_DEPTH                              # the K reads in flight on entry: they complete first, in order
+    out += check_rescale(uid, cb, True)
+    out += v_address_ops(S_R0)                          # V^T addresses of tile t (the previous iteration set them too; kept explicit)
+    for n in range(32):
+        if n == 16:
+            out += [f"s_waitcnt vmcnt({DMA_PER_TILE})", "s_barrier"]
+        if n < 16:
+            out.extend(plan[n])
+            out.append("s_nop 1")                       # no MFMAs here to space a v_exp from the conversion that reads it
+            k = n + RING_DEPTH
+            if k >= 16:
+                rg.read(out, k, items[k], k)
+            continue
+        if n % 2 == 0:
+            rg.wait(out, n + 1)
+        first, last = dma[n - 17] if 17 <= n < 17 + DMA_PER_TILE else ([], [])
+        out.extend(first)
+        spread(out, items[n][1](ring(n)), plan[n])
+        k = n + RING_DEPTH
+        if k < 32:
+            rg.read(out, k, items[k], k)
+        out.extend(last)
+    out += [f"s_mov_b32 {S_TMP}, {S_R0}", f"s_mov_b32 {S_R0}, {S_R1}", f"s_mov_b32 {S_R1}, {S_R2}", f"s_mov_b32 {S_R2}, {S_R3}",
+            f"s_mov_b32 {S_R3}, {S_R4}", f"s_mov_b32 {S_R4}, {S_TMP}",
+            f"s_add_i32 {S_T}, {S_T}, 1",
+            f"s_cmp_ge_i32 {S_T}, %[nt]",
+            "s_cbranch_scc1 .Lend_%=",
+            "s_branch .Lidle_%="]
+    return out
+
+
 def select(cb):
     """Top of iteration t: leave after the last tile; tiles that need the key mask go out of line."""
     return [f".Ltop_{cb}_%=:",
@@ -461,9 +507,11 @@ def select(cb):
             "s_cbranch_scc1 .Lend_%=",
             f"s_cmp_ge_i32 {S_KEY0}, %[whx]",
             "s_cbranch_scc1 .Lidle_%=",
+            f"s_add_i32 {S_TMP}, {S_KEY0}, 64",
+            f"s_cmp_ge_i32 {S_TMP}, %[whx]",
+            f"s_cbranch_scc1 .Llast_{cb}_%=",
             f"s_cmp_lt_i32 {S_KEY0}, %[pad]",
             f"s_cbranch_scc1 .Lmasked_{cb}_%=",
-            f"s_add_i32 {S_TMP}, {S_KEY0}, 64",
             f"s_cmp_gt_i32 {S_TMP}, %[whm]",
             f"s_cbranch_scc1 .Lmasked_{cb}_%="]
 
@@ -513,6 +561,8 @@ def program():
     out += select(0) + body(0, False) + select(1) + body(1, False) + ["s_branch .Ltop_0_%="]
     out += [".Lmasked_0_%=:"] + body(0, True) + ["s_branch .Ltop_1_%="]
     out += [".Lmasked_1_%=:"] + body(1, True) + ["s_branch .Ltop_0_%="]
+    out += [".Llast_0_%=:"] + body_last(0)
+    out += [".Llast_1_%=:"] + body_last(1)
     out += idle_loop()
     out += epilogue()
     return out
