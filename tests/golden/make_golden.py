@@ -104,6 +104,68 @@ def main():
     np.savez_compressed(OUT / "layer_ops.npz", x=bits(x), residual=bits(r), weight=bits(w), eps=np.float32(1e-6),
                         normed=bits(y), new_residual=bits(nr), normed_no_residual=bits(y0),
                         gate_up=bits(gu), act=bits(oracle.silu_and_mul(gu)))
+    # ---- sampling: top-k 20 then top-p 0.8 on 8 rows of 600 logits, then the step's Gumbel draw from (seed, offset);
+    #      a generator of its own, so that the fixtures above keep their bytes
+    g2 = torch.Generator().manual_seed(777002)
+    V2 = 600
+    lg = (torch.randn(2, 4, V2, generator=g2) * 2.5).bfloat16()
+    t2 = np.array([0.8, 1.25], dtype=np.float32)
+    seed, offset = 2 ** 33 + 12345, 2 ** 32 + 7
+    x64 = lg.to(torch.float64).numpy().reshape(8, V2)
+    T8 = np.repeat(t2.astype(np.float64), 4)
+    kept_k = np.isfinite(oracle.filter_logits(x64, top_k=20))
+    for r in range(8):                                           # no cumulative probability within 1e-3 of p: not a rounding matter
+        vals = np.sort(x64[r][kept_k[r]])[::-1] / T8[r]
+        pr = np.exp(vals - vals[0])
+        assert np.abs(np.cumsum(pr / pr.sum()) - 0.8).min() > 1e-3, "fixture sits on the top-p boundary: change the seed"
+    filt = oracle.filter_logits(x64, top_k=20, top_p=0.8, temperatures=T8)
+    noise = oracle.gumbel_noise(8, V2, seed, offset)
+    sx0, sp = oracle.confidence_argmax(filt.reshape(2, 4, V2), t2, noise.reshape(2, 4, V2))
+    noisy = np.where(np.isfinite(filt), (filt.astype(np.float32) / T8[:, None].astype(np.float32)).astype(np.float64) + noise, -np.inf)
+    top2 = np.sort(noisy, axis=-1)[:, -2:]
+    assert np.all(top2[:, 1] - top2[:, 0] > 1e-3), "fixture sits on a tie of the noisy argmax: change the seed"
+    np.savez_compressed(OUT / "sampling.npz", logits=bits(lg), temperatures=t2, top_k=np.int32(20), top_p=np.float32(0.8),
+                        kept=np.isfinite(filt).astype(np.uint8), seed=np.uint64(seed), offset=np.uint64(offset),
+                        noise=noise.astype(np.float32), x0=sx0.astype(np.int64), x0_p=sp.astype(np.float32))
+
+    # ---- block state on the device: 5 lanes of 8 positions, pages of 16 tokens
+    rng = np.random.default_rng(991)
+    S8, page16, mask_id2 = 8, 16, 99
+    lens5 = np.array([16, 40, 8, 0, 24], dtype=np.int32)
+    phase5 = np.array([1, 2, 1, 0, 2], dtype=np.int32)          # denoising, caching, denoising, idle, caching
+    bt5 = np.array([[3, 7, -1, -1], [1, 0, 5, 9], [2, 6, -1, -1], [-1, -1, -1, -1], [4, 8, 10, -1]], dtype=np.int32)
+    pos5, slots5, ctx5 = oracle.block_prepare(lens5, phase5, bt5, page16, S8)
+    tok5 = rng.integers(0, 90, (5, S8)).astype(np.int64)
+    tok5[0, [1, 4, 6]] = mask_id2
+    tok5[2, :] = mask_id2
+    tok5[1, 3] = 55                                              # lane 1 (caching) holds its stop token
+    rows5, n5 = oracle.masked_rows(tok5, phase5, mask_id2, 16)
+    transfer5 = np.zeros((5, S8), dtype=np.uint8)
+    transfer5[0, [1, 4, 6]] = 1                                  # lane 0 commits its last three positions -> caching
+    transfer5[2, [0, 5]] = 1
+    tok_sel = tok5.copy()
+    tok_sel[0, [1, 4, 6]] = [11, 12, 13]
+    tok_sel[2, [0, 5]] = [21, 22]
+    step_map5 = rng.integers(0, 3, (5, S8)).astype(np.int32)
+    step5 = np.array([3, 8, 0, 0, 8], dtype=np.int32)
+    first5 = np.array([8, 16, 8, 0, 8], dtype=np.int32)
+    maxnew5 = np.array([64, 64, 64, 64, 24], dtype=np.int32)    # lane 4 reaches its budget with this block
+    stop5 = np.array([[-1, -1], [55, -1], [-1, -1], [-1, -1], [77, -1]], dtype=np.int64)
+    a_tok, a_map, a_step, a_phase, a_lens, appended, status = oracle.block_advance(
+        tok_sel, transfer5, step_map5, step5, phase5, lens5, first5, maxnew5, stop5, mask_id2)
+    out_tok = np.full((5, 64), -1, dtype=np.int64)
+    out_step = np.full((5, 64), -1, dtype=np.int32)
+    for b, ap in enumerate(appended):
+        if ap is not None:
+            at = int(lens5[b] - first5[b])
+            out_tok[b, at:at + S8], out_step[b, at:at + S8] = ap
+    st = np.array([[s[0], lens5[b] if s[1] is None else s[1], s[2], s[3]] for b, s in enumerate(status)], dtype=np.int32)
+    np.savez_compressed(OUT / "block_state.npz", lens=lens5, phase=phase5, block_table=bt5, page=np.int32(page16), block_len=np.int32(S8),
+                        positions=pos5, slot_mapping=slots5, context_lens=ctx5, mask_id=np.int64(mask_id2),
+                        tokens=tok5, rows=rows5, n_rows=np.int32(n5), tokens_selected=tok_sel, transfer=transfer5,
+                        step_map=step_map5, step=step5, first_len=first5, max_new=maxnew5, stop_ids=stop5,
+                        tokens_after=a_tok, step_map_after=a_map, step_after=a_step, phase_after=a_phase, lens_after=a_lens,
+                        out_tokens=out_tok, out_steps=out_step, status=st)
     for f in sorted(OUT.glob("*.npz")):
         print(f.name, f.stat().st_size, "bytes")
 

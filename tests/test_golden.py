@@ -60,7 +60,88 @@ def test_oracle_reproduces_layer_op_fixtures():
     assert torch.equal(oracle.silu_and_mul(bf16(f["gate_up"])), bf16(f["act"]))
 
 
+def test_oracle_reproduces_sampling_and_block_state_fixtures():
+    f = load("sampling.npz")
+    x = bf16(f["logits"]).to(torch.float64).numpy().reshape(8, -1)
+    T8 = np.repeat(f["temperatures"].astype(np.float64), 4)
+    filt = oracle.filter_logits(x, top_k=int(f["top_k"]), top_p=float(f["top_p"]), temperatures=T8)
+    assert np.array_equal(np.isfinite(filt).astype(np.uint8), f["kept"])
+    assert 1 <= f["kept"].sum(1).min() and f["kept"].sum(1).max() <= int(f["top_k"])
+    noise = oracle.gumbel_noise(8, x.shape[1], int(f["seed"]), int(f["offset"]))
+    assert np.array_equal(noise.astype(np.float32), f["noise"])
+    x0, p = oracle.confidence_argmax(filt.reshape(2, 4, -1), f["temperatures"], noise.reshape(2, 4, -1))
+    assert np.array_equal(x0, f["x0"]) and np.allclose(p, f["x0_p"], rtol=1e-6)
+    assert f["kept"].reshape(2, 4, -1)[np.arange(2)[:, None], np.arange(4)[None], x0].all()      # every drawn token survived the filter
+    b = load("block_state.npz")
+    pos, slots, ctx = oracle.block_prepare(b["lens"], b["phase"], b["block_table"], int(b["page"]), int(b["block_len"]))
+    assert np.array_equal(pos, b["positions"]) and np.array_equal(slots, b["slot_mapping"]) and np.array_equal(ctx, b["context_lens"])
+    rows, n = oracle.masked_rows(b["tokens"], b["phase"], int(b["mask_id"]), len(b["rows"]))
+    assert np.array_equal(rows, b["rows"]) and n == int(b["n_rows"])
+    tok, smap, step, phase, lens, appended, status = oracle.block_advance(
+        b["tokens_selected"], b["transfer"], b["step_map"], b["step"], b["phase"], b["lens"], b["first_len"], b["max_new"],
+        b["stop_ids"], int(b["mask_id"]))
+    assert np.array_equal(tok, b["tokens_after"]) and np.array_equal(smap, b["step_map_after"]) and np.array_equal(step, b["step_after"])
+    assert np.array_equal(phase, b["phase_after"]) and np.array_equal(lens, b["lens_after"])
+    # the fixture walks every transition: denoising -> caching, caching -> idle by stop token and by budget, idle stays idle
+    assert b["phase"].tolist() == [1, 2, 1, 0, 2] and b["phase_after"].tolist() == [2, 0, 1, 0, 0]
+
+
 # ----------------------------------------------------------------------------- GPU: HIP path == fixtures
+@pytest.mark.gpu
+def test_hip_sampling_matches_fixtures(dev):
+    import mdx
+    f = load("sampling.npz")
+    logits = bf16(f["logits"]).to(dev)
+    temps = torch.from_numpy(f["temperatures"]).to(dev)
+    V = logits.shape[-1]
+    filt = mdx.filter_logits(logits, top_k=int(f["top_k"]), top_p=float(f["top_p"]), temperatures=temps)
+    assert np.array_equal(torch.isfinite(filt.float()).cpu().numpy().reshape(8, V).astype(np.uint8), f["kept"])
+    assert torch.equal(filt[torch.isfinite(filt.float())], logits[torch.isfinite(filt.float())])
+    noise = mdx.gumbel_noise(8, V, int(f["seed"]), int(f["offset"]), device=dev)
+    np.testing.assert_allclose(noise.cpu().numpy(), f["noise"], rtol=0, atol=3e-6)
+    x0, p = mdx.confidence_argmax(filt, temps, seed=int(f["seed"]), offset=int(f["offset"]))
+    assert np.array_equal(x0.cpu().numpy(), f["x0"])
+    np.testing.assert_allclose(p.cpu().numpy(), f["x0_p"], rtol=3e-5)
+
+
+@pytest.mark.gpu
+def test_hip_block_state_matches_fixtures(dev):
+    import mdx
+    b = load("block_state.npz")
+    L = mdx.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    d = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)      # noqa: E731
+    bs, S, width = len(b["lens"]), int(b["block_len"]), b["block_table"].shape[1]
+    lens, phase, bt = d(b["lens"]), d(b["phase"]), d(b["block_table"])
+    pos = torch.empty(bs, S, dtype=torch.int64, device=dev)
+    slots = torch.empty(bs, S, dtype=torch.int32, device=dev)
+    ctx = torch.empty(bs, dtype=torch.int32, device=dev)
+    assert L.mdx_block_prepare(lens.data_ptr(), phase.data_ptr(), bt.data_ptr(), width, width, int(b["page"]), S,
+                               pos.data_ptr(), slots.data_ptr(), ctx.data_ptr(), bs, stream) == 0
+    assert np.array_equal(pos.cpu().numpy(), b["positions"]) and np.array_equal(slots.cpu().numpy(), b["slot_mapping"])
+    assert np.array_equal(ctx.cpu().numpy(), b["context_lens"])
+    cap = len(b["rows"])
+    rows = torch.empty(cap, dtype=torch.int64, device=dev)
+    n = torch.empty(1, dtype=torch.int32, device=dev)
+    tok = d(b["tokens"])
+    assert L.mdx_masked_rows(tok.data_ptr(), phase.data_ptr(), int(b["mask_id"]), bs, S, rows.data_ptr(), cap, n.data_ptr(), stream) == 0
+    assert np.array_equal(rows.cpu().numpy(), b["rows"]) and int(n.item()) == int(b["n_rows"])
+    tok2, tr, smap, step = d(b["tokens_selected"]), d(b["transfer"]), d(b["step_map"]), d(b["step"])
+    first, mx, stop = d(b["first_len"]), d(b["max_new"]), d(b["stop_ids"])
+    out_tok = torch.full((bs, 64), -1, dtype=torch.int64, device=dev)
+    out_step = torch.full((bs, 64), -1, dtype=torch.int32, device=dev)
+    status = torch.zeros(bs, 4, dtype=torch.int32, device=dev)
+    assert L.mdx_block_advance(tok2.data_ptr(), tr.data_ptr(), smap.data_ptr(), step.data_ptr(), phase.data_ptr(), lens.data_ptr(),
+                               first.data_ptr(), mx.data_ptr(), stop.data_ptr(), stop.shape[1], out_tok.data_ptr(), out_step.data_ptr(),
+                               64, status.data_ptr(), int(b["mask_id"]), bs, S, stream) == 0
+    torch.cuda.synchronize()
+    live = b["phase"] != 0
+    assert np.array_equal(tok2.cpu().numpy(), b["tokens_after"]) and np.array_equal(smap.cpu().numpy(), b["step_map_after"])
+    assert np.array_equal(step.cpu().numpy()[live], b["step_after"][live])
+    assert np.array_equal(phase.cpu().numpy(), b["phase_after"]) and np.array_equal(lens.cpu().numpy(), b["lens_after"])
+    assert np.array_equal(out_tok.cpu().numpy(), b["out_tokens"]) and np.array_equal(out_step.cpu().numpy(), b["out_steps"])
+    st = status.cpu().numpy()
+    assert np.array_equal(st[live], b["status"][live]) and st[~live][:, 0].tolist() == [0] * int((~live).sum())
 @pytest.mark.gpu
 def test_hip_attention_matches_fixtures(dev):
     import mdx
