@@ -616,7 +616,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "config 3: one prefill pass of the attention layer (store_kvcache + staircase "
-                               "block-prefill attention) over 8 packed sequences",
+                               "block-prefill attention) over 8 packed sequences; mdx.Attention launches the store on a second stream beside "
+                               "the attention kernel and joins both before it returns",
                    "seq_lens": host3["lens"], "total_tokens": work3["tokens"], "block": S, "num_q_heads": HQ,
                    "num_kv_heads": HKV, "head_dim": D, "page_size": PAGE, "visible_pairs": work3["pairs"],
                    "algorithmic_gflop": round(work3["flops"] / 1e9, 2)},

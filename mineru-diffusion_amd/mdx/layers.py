@@ -8,6 +8,18 @@ from .context import get_context
 from .ops import flash_attn_with_kvcache, sparse_attn_varlen, store_kvcache_maybe4d, unmask_step
 
 
+_side_streams: dict = {}
+
+
+def _side_stream(device: torch.device) -> torch.cuda.Stream:
+    """One extra stream per device (default priority) for work that may run beside the caller's stream."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    stream = _side_streams.get(index)
+    if stream is None:
+        stream = _side_streams[index] = torch.cuda.Stream(device=index)
+    return stream
+
+
 class Attention(nn.Module):
     """nanovllm/layers/sdar_attention.py:19-57: store the step's K/V into the paged cache,
     then staircase attention over the packed prompt (prefill) or non-causal attention of
@@ -24,18 +36,28 @@ class Attention(nn.Module):
     def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
         context = get_context()
         k_cache, v_cache = self.k_cache, self.v_cache
-        if k_cache.numel() and v_cache.numel():
-            store_kvcache_maybe4d(k, v, k_cache, v_cache, context.slot_mapping)
+        have_cache = bool(k_cache.numel() and v_cache.numel())
         if context.is_prefill:
+            # The prefill attention reads k / v, not the cache: the store is independent of it and runs beside it on a
+            # second stream (its small workgroups fill the gaps between the attention kernel's, which own whole CUs:
+            # config 3, 0.820 -> 0.808 ms for the pair).  The caller's stream waits for both before it goes on.
+            main = torch.cuda.current_stream(q.device)
+            side = _side_stream(q.device) if have_cache else None
+            if side is not None:
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    store_kvcache_maybe4d(k, v, k_cache, v_cache, context.slot_mapping)
             o = sparse_attn_varlen(q, k, v, cu_seqlens_q=context.cu_seqlens_q, cu_seqlens_k=context.cu_seqlens_k,
                                    staircase_size=context.block_size,
                                    max_seqlen=context.max_seqlen_k or None, softmax_scale=self.scale)
-            o = o.flatten(1)
-        else:
-            o = flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=context.context_lens,
-                                        block_table=context.block_tables, softmax_scale=self.scale, causal=False)
-            o = o.flatten(2)
-        return o
+            if side is not None:
+                main.wait_stream(side)
+            return o.flatten(1)
+        if have_cache:
+            store_kvcache_maybe4d(k, v, k_cache, v_cache, context.slot_mapping)
+        o = flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=context.context_lens,
+                                    block_table=context.block_tables, softmax_scale=self.scale, causal=False)
+        return o.flatten(2)
 
 
 class Sampler(nn.Module):
