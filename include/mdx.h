@@ -80,9 +80,12 @@ int mdx_store_kvcache(const void* key, const void* value,
  * sizes the grid, and rows of a longer sequence beyond it are never computed
  * (their o rows keep what they held; the lengths are on the device, so the
  * call cannot check this).  total_tokens is always a valid bound; the
- * reference interface has no such argument.  Supported: d == 128, dtype
- * MDX_BF16 or MDX_F16 (the reference kernel takes q's dtype, :179-197; fp16
- * runs the one-head-per-wavefront kernel, about 0.8 x the bf16 rate).
+ * reference interface has no such argument.  Supported: d a multiple of 16
+ * up to 128 (the reference kernel takes BLOCK_DMODEL = head_dim, :183; widths
+ * below 128 run as 128 with zero padding, in the one-head-per-wavefront
+ * kernel, and only d columns of o are written), dtype MDX_BF16 or MDX_F16
+ * (the reference kernel takes q's dtype, :179-197; fp16 runs the one-head
+ * kernel too, about 0.8 x the bf16 rate).
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                               int64_t q_stride_t, int64_t q_stride_h,
@@ -115,7 +118,9 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * kernel picks it from the lengths); its size comes from
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
  * contents need no initialisation.
- * Supported: d == 128, Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0, MDX_BF16 or MDX_F16.
+ * Supported: d a multiple of 16 up to 128 (narrower heads are padded with zeros on the way into LDS; the
+ * partials keep their 128-wide layout), Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0,
+ * MDX_BF16 or MDX_F16.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
                                              int32_t num_kv_heads, int32_t head_dim,

@@ -110,8 +110,10 @@ struct WaveState {
 // n0 .. n0+NSUB*32-1 of tiles with row pitch kLdsPitch.
 
 // S^T = K Q^T.  q[h][ks] are the B-operand fragments of Q^T for d = 16ks .. 16ks+15.
+// Columns from `width` on (a multiple of 16) are zeros on both sides and skipped.
 template <typename E, int NH, int NSUB>
-__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const typename Elem16<E>::vec8 (&q)[NH][8], f32x16 (&s)[NH][NSUB], int lane)
+__device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const typename Elem16<E>::vec8 (&q)[NH][8], f32x16 (&s)[NH][NSUB], int lane,
+                                         int width = kHeadDim)
 {
     typedef typename Elem16<E>::vec8 vec8;
     const int H = lane >> 5, r = lane & 31;
@@ -124,6 +126,7 @@ __device__ __forceinline__ void qk_phase(const char* lds_k, int n0, const typena
     const char* kbase = lds_k + (n0 + key_of_mfma_row(r)) * kLdsPitch + H * 16;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
+        if (ks * 16 >= width) break;
 #pragma unroll
         for (int u = 0; u < NSUB; ++u) {
             const vec8 kf = *reinterpret_cast<const vec8*>(kbase + u * 32 * kLdsPitch + ks * 32);
@@ -194,8 +197,10 @@ __device__ __forceinline__ void softmax_phase(f32x16 (&s)[NH][NSUB], typename El
 
 // O^T += V^T P^T.  The lane supplies the row address for the transposing read:
 // row 4*(i'/4) + 2H (+q), d chunk i'%4, with i' = lane % 16.
+// O^T tiles whose 32 rows all lie beyond `width` stay zero and are skipped.
 template <typename E, int NH, int NSUB>
-__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const typename Elem16<E>::vec8 (&p)[NH][NSUB][2], WaveState<NH>& st, int lane)
+__device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const typename Elem16<E>::vec8 (&p)[NH][NSUB][2], WaveState<NH>& st, int lane,
+                                         int width = kHeadDim)
 {
     typedef typename Elem16<E>::vec8 vec8;
     const int H = lane >> 5, ip = lane & 15, gi = (lane >> 4) & 1;
@@ -206,6 +211,7 @@ __device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const typena
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
+                if (dt * 32 >= width) break;
                 const lds_char* a = vbase + (u * 32 + t * 16) * kLdsPitch + dt * 64;
                 const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)a);
                 const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(a + kLdsPitch));
@@ -220,25 +226,26 @@ __device__ __forceinline__ void pv_phase(const char* lds_v, int n0, const typena
 // All three phases back to back.
 template <typename E, int NH, int NSUB, bool MASK>
 __device__ __forceinline__ void attn_step(const char* lds_k, const char* lds_v, int n0, const typename Elem16<E>::vec8 (&q)[NH][8],
-                                          WaveState<NH>& st, float c, int lane, int key_abs0, int key_lo, int key_hi)
+                                          WaveState<NH>& st, float c, int lane, int key_abs0, int key_lo, int key_hi, int width = kHeadDim)
 {
     f32x16 s[NH][NSUB];
     typename Elem16<E>::vec8 p[NH][NSUB][2];
-    qk_phase<E, NH, NSUB>(lds_k, n0, q, s, lane);
+    qk_phase<E, NH, NSUB>(lds_k, n0, q, s, lane, width);
     softmax_phase<E, NH, NSUB, MASK>(s, p, st, c, lane, key_abs0, key_lo, key_hi);
-    pv_phase<E, NH, NSUB>(lds_v, n0, p, st, lane);
+    pv_phase<E, NH, NSUB>(lds_v, n0, p, st, lane, width);
 }
 
 // d index held by accumulator register i of O^T tile dt in half-wave H.
 __device__ __forceinline__ int d_of_reg(int dt, int i, int H) { return dt * 32 + 8 * (i >> 2) + 4 * H + (i & 3); }
 
 // Loads the Q^T B-operand fragments of one head for this lane's query row
-// (row pointer may be null: zeros).  q_row points at Q[query, head, 0].
+// (row pointer may be null: zeros).  q_row points at Q[query, head, 0]; a head narrower than 128
+// (width: a multiple of 16) is padded with zeros.
 template <typename V8>
-__device__ __forceinline__ void load_q(V8 (&q)[8], const __bf16* q_row, int H) {
+__device__ __forceinline__ void load_q(V8 (&q)[8], const __bf16* q_row, int H, int width = kHeadDim) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-        if (q_row) {
+        if (q_row && ks * 16 < width) {
             q[ks] = *reinterpret_cast<const V8*>(q_row + ks * 16 + H * 8);
         } else {
 #pragma unroll

@@ -70,6 +70,7 @@ struct PagedParams {
     int64_t num_pages;
     int chunk, nsplit;                              // keys per split, max splits per sequence
     int num_q_heads;
+    int head_dim;                                   // <= 128, a multiple of 16: columns beyond it are zeros in LDS and never stored
     float c;                                        // scale * log2(e)
     float* part_o; float* part_ml;                  // [bs, Hq, nsplit, 32, 128] and [bs, Hq, nsplit, 2, 32]
     // non-null: the attention kernel picks the split size (>= chunk) from the lengths and leaves it
@@ -88,6 +89,7 @@ struct PagedParams {
 template <typename E, bool AGENT>
 __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, int nv)
 {
+    if (c * 16 >= P.head_dim) return;
     const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
     float M = kMinusBig, Lsum = 0.f;
     float acc[16];
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         if (split == 0) {
             for (int e = tid; e < P.sq * HPW * (kHeadDim / 8); e += kThreads) {
                 const int d8 = e % (kHeadDim / 8), h = (e / (kHeadDim / 8)) % HPW, s = e / (kHeadDim / 8) / HPW;
-                *reinterpret_cast<u32x4*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)(hg * HPW + h) * P.o_sh + d8 * 8) = u32x4{0, 0, 0, 0};
+                if (d8 * 8 < P.head_dim) *reinterpret_cast<u32x4*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)(hg * HPW + h) * P.o_sh + d8 * 8) = u32x4{0, 0, 0, 0};
             }
         }
         return;
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
 
     const bool row_ok = r < P.sq;
     typename Elem16<E>::vec8 q[1][8];
-    load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H);
+    load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H, P.head_dim);
 
     WaveState<1> st;
     st.init();
@@ -252,7 +254,9 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         unsigned row_ok;       // bit p: this thread's row of pass p holds a real key
         unsigned pass_ok;      // bit p (uniform): pass p lies on a valid page inside the context
     };
-    const int64_t safe_off = (int64_t)trow * P.c_st + (int64_t)kvh * P.c_sh + chunk * 8;
+    // (a thread whose 16-byte chunk lies beyond a narrow head reads the head's last chunk instead; zeroed like a row past the end)
+    const bool col_ok = chunk * 8 < P.head_dim;
+    const int64_t safe_off = (int64_t)trow * P.c_st + (int64_t)kvh * P.c_sh + min(chunk * 8, P.head_dim - 8);
     auto fetch = [&](Staged& sg, int t) {
         const int key0 = key_begin + t * kTileKeys;
         sg.row_ok = 0;
@@ -269,7 +273,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             sg.regs.k[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.k_cache + off));
             sg.regs.v[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(P.v_cache + off));
             sg.pass_ok |= (ok ? 1u : 0u) << p;
-            sg.row_ok |= ((ok && kp + trow < key_end) ? 1u : 0u) << p;
+            sg.row_ok |= ((ok && col_ok && kp + trow < key_end) ? 1u : 0u) << p;
         }
     };
     unsigned tile_pass_ok[2] = {0, 0};                 // pass_ok of the tile sitting in LDS buffer 0 / 1
@@ -373,7 +377,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
                 typename Elem16<E>::vec4 out;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
-                *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+                if (d_of_reg(dt, 4 * g, H) < P.head_dim) *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
             }
         return;
     }
@@ -502,7 +506,8 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && sq >= 0 && max_pages >= 0 && num_pages >= 0, MDX_EINVAL, "paged_block_attn: negative size");
     MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "paged_block_attn: dtype %d (bf16 or fp16)", dtype);
-    MDX_REQUIRE(head_dim == kHeadDim, MDX_EUNSUPPORTED, "paged_block_attn: head_dim %d (only 128)", head_dim);
+    MDX_REQUIRE(head_dim >= 16 && head_dim <= kHeadDim && head_dim % 16 == 0, MDX_EUNSUPPORTED,
+                "paged_block_attn: head_dim %d (multiples of 16 up to 128)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "paged_block_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
     MDX_REQUIRE(sq <= kMaxSq, MDX_EUNSUPPORTED, "paged_block_attn: %d queries per sequence (max %d)", sq, kMaxSq);
@@ -534,6 +539,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     P.chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size, &device_span);
     P.nsplit = nsplit_of(max_pages, page_size, P.chunk);
     P.num_q_heads = num_q_heads;
+    P.head_dim = head_dim;
     P.c = scale * kLog2e;
     P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr; P.arrive = nullptr;
     if (P.nsplit > 1) {

@@ -43,6 +43,7 @@ struct StaircaseParams {
     int total_tokens;
     int batch, n_row_groups, num_q_heads, num_kv_heads;
     int log2_s;
+    int head_dim;                                              // <= 128, a multiple of 16
     float c;                                                   // scale * log2(e)
 };
 
@@ -101,9 +102,12 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
     return true;
 }
 
-template <typename E>
+// NARROW: head_dim below 128 (a multiple of 16).  Rows of q, k, v are then padded with zeros on their way into
+// registers and LDS, products over the padding are skipped, and only head_dim columns of o are written.
+template <typename E, bool NARROW>
 __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const StaircaseParams P)
 {
+    const int width = NARROW ? P.head_dim : kHeadDim;
     __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
     __shared__ __attribute__((aligned(16))) char lds_vbuf[2][kTileBytes];
 
@@ -133,7 +137,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
     typename Elem16<E>::vec8 q[1][8];
-    load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H);
+    load_q(q[0], row_ok ? P.q + tok * P.q_st + (int64_t)head * P.q_sh : nullptr, H, width);
 
     // exclusive key limit (padded coordinates) of this lane's row, and the wavefront's extremes
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
@@ -150,6 +154,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     // Thread-private row pointers walk down the sequence one tile per fetch; rows outside the
     // sequence (only possible in the first and last tiles) are never dereferenced.
     const int chunk = tid & 15, trow = tid >> 4;
+    const bool col_ok = !NARROW || chunk * 8 < width;          // this thread's 16-byte chunk exists in a row
     constexpr int kPasses = TileRegs<kTileKeys, kThreads>::kPasses;
     constexpr int kRowsPerPass = kThreads / 16;
     const int64_t row0 = (int64_t)seq0 - pad + trow;          // token of LDS row `trow` of tile 0
@@ -162,10 +167,10 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 #pragma unroll
         for (int p = 0; p < kPasses; ++p) {
             const int jp = t * kTileKeys + trow + kRowsPerPass * p;
-            if (interior || (jp >= pad && jp < Lp)) {
+            if (col_ok && (interior || (jp >= pad && jp < Lp))) {
                 regs.k[p] = *reinterpret_cast<const u32x4*>(kcur + p * k_pass);
                 regs.v[p] = *reinterpret_cast<const u32x4*>(vcur + p * v_pass);
-            } else {                           // keys outside the sequence: zero rows, masked below
+            } else {                           // keys outside the sequence: zero rows, masked below (or padding columns)
                 regs.k[p] = u32x4{0, 0, 0, 0};
                 regs.v[p] = u32x4{0, 0, 0, 0};
             }
@@ -184,11 +189,11 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         const int key0 = t * kTileKeys;
         if (key0 < wave_hi) {
             if (key0 >= pad && key0 + kTileKeys <= wave_hi_min) {
-                attn_step<E, 1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 2, false>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi, width);
             } else if (key0 + 32 < wave_hi) {
-                attn_step<E, 1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 2, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi, width);
             } else {
-                attn_step<E, 1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi);
+                attn_step<E, 1, 1, true>(lds_k, lds_v, 0, q, st, P.c, lane, key0, pad, key_hi, width);
             }
         }
         if (t + 1 < n_tiles) {
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
             typename Elem16<E>::vec4 out;
 #pragma unroll
             for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
-            *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
+            if (!NARROW || d_of_reg(dt, 4 * g, H) < width) *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
         }
 }
 
@@ -331,7 +336,8 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(batch >= 0 && total_tokens >= 0 && max_seqlen >= 0, MDX_EINVAL, "staircase_attn: negative size");
     MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (bf16 or fp16)", dtype);
-    MDX_REQUIRE(head_dim == kHeadDim, MDX_EUNSUPPORTED, "staircase_attn: head_dim %d (only 128)", head_dim);
+    MDX_REQUIRE(head_dim >= 16 && head_dim <= kHeadDim && head_dim % 16 == 0, MDX_EUNSUPPORTED,
+                "staircase_attn: head_dim %d (multiples of 16 up to 128)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "staircase_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
     int log2_s = -1;
@@ -359,6 +365,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.n_row_groups = (int)((max_l + staircase_size - 1 + rows_per_wg - 1) / rows_per_wg);
     P.num_q_heads = num_q_heads;
     P.num_kv_heads = num_kv_heads;
+    P.head_dim = head_dim;
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
     // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence
@@ -371,7 +378,8 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     // prologue, epilogue: 10 us) is then most of its time, while two one-head workgroups share a CU and hide each
     // other's (64 x 600 tokens: 0.237 against 0.259 ms, 16 x 300: 0.028 against 0.035; equal at 1100 tokens, and
     // from there on the pair kernel wins: 1.3 x at 8 x 4096).
-    const bool pairs = dtype == MDX_BF16 && max_l > 640 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
+    const bool narrow = head_dim < kHeadDim;                   // one-head kernel, rows padded with zeros
+    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 640 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
@@ -381,9 +389,11 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
         MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
         staircase_pair_kernel<<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
     } else if (dtype == MDX_F16) {
-        staircase_attn_kernel<_Float16><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+        if (narrow) staircase_attn_kernel<_Float16, true><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+        else        staircase_attn_kernel<_Float16, false><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     } else {
-        staircase_attn_kernel<__bf16><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+        if (narrow) staircase_attn_kernel<__bf16, true><<<(unsigned)grid, kThreads, 0, stream>>>(P);
+        else        staircase_attn_kernel<__bf16, false><<<(unsigned)grid, kThreads, 0, stream>>>(P);
     }
     return mdx::check_launch("staircase_attn");
 }

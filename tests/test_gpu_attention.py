@@ -424,3 +424,58 @@ def test_fp16_prefill_and_decode(dev, hq, hkv):
         od2 = mdx.flash_attn_with_kvcache(qd.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens_d.to(dev), block_table=bt.to(dev),
                                           softmax_scale=scale, causal=False, counters=False)
         assert torch.equal(od.view(torch.int16), od2.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [16, 32, 64, 96, 112])
+def test_narrow_heads_prefill_and_decode(dev, d, dtype):
+    """The reference kernel takes BLOCK_DMODEL = head_dim (block_prefill_attention_v2.py:183) and flash-attn any head
+    width: heads narrower than 128 (multiples of 16) through both attention calls against the fp32 oracle, scale
+    d^-0.5, q / k / v read in place from a fused projection (rows 16-byte aligned but not 256-byte wide), an odd and
+    an even head ratio, split and unsplit paged sequences, and the columns of o beyond no head's width left alone."""
+    import mdx
+    g = torch.Generator().manual_seed(9000 + d)
+    for hq, hkv in ((4, 2), (3, 1)):
+        lens = [333, 64, 1000, 31]
+        N = sum(lens)
+        fused = torch.randn(N, (hq + 2 * hkv) * d, generator=g).to(dtype)
+        q = fused[:, :hq * d].unflatten(-1, (hq, d))
+        k = fused[:, hq * d:(hq + hkv) * d].unflatten(-1, (hkv, d))
+        v = fused[:, (hq + hkv) * d:].unflatten(-1, (hkv, d))
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        fd = fused.to(dev)
+        qd, kd, vd = fd[:, :hq * d].unflatten(-1, (hq, d)), fd[:, hq * d:(hq + hkv) * d].unflatten(-1, (hkv, d)), fd[:, (hq + hkv) * d:].unflatten(-1, (hkv, d))
+        for bound in (None, 2048):
+            o = mdx.sparse_attn_varlen(qd, kd, vd, cu.to(dev), cu.to(dev), 32, max_seqlen=bound)
+            assert o.shape == (N, hq, d) and o.dtype == dtype
+            ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
+            err = (o.float().cpu() - ref).abs().max().item()
+            assert err < TOL, f"prefill d={d} hq={hq}: max-abs {err}"
+        for ctxs in ([700, 4128, 33, 0], [2300] * 4):
+            qp, kc, vc, bt, lens_d = _paged_inputs(g, ctxs, hq=hq, hkv=hkv, d=d, pool=40)
+            qp, kc, vc = qp.to(dtype), kc.to(dtype), vc.to(dtype)
+            scale = 1 / math.sqrt(d)
+            kwargs = dict(cache_seqlens=lens_d.to(dev), block_table=bt.to(dev), softmax_scale=scale, causal=False)
+            od = mdx.flash_attn_with_kvcache(qp.to(dev), kc.to(dev), vc.to(dev), **kwargs)
+            refd = oracle.paged_block_attn(qp, kc, vc, bt, lens_d, scale)
+            err = (od.float().cpu() - refd).abs().max().item()
+            assert err < TOL, f"paged d={d} hq={hq} ctxs={ctxs}: max-abs {err}"
+            od2 = mdx.flash_attn_with_kvcache(qp.to(dev), kc.to(dev), vc.to(dev), **kwargs, counters=False)
+            assert torch.equal(od.view(torch.int16), od2.view(torch.int16))
+    # o embedded in a wider buffer: what lies beyond the head's width stays as it was
+    L = mdx._lib.lib()
+    hq, hkv = 4, 2
+    q1 = torch.randn(100, hq, d, generator=g).to(dtype).to(dev)
+    k1 = torch.randn(100, hkv, d, generator=g).to(dtype).to(dev)
+    v1 = torch.randn(100, hkv, d, generator=g).to(dtype).to(dev)
+    wide = torch.full((100, hq, 128), 7.0, dtype=dtype, device=dev)
+    cu1 = torch.tensor([0, 100], dtype=torch.int32, device=dev)
+    rc = L.mdx_staircase_attn_varlen(q1.data_ptr(), k1.data_ptr(), v1.data_ptr(), wide.data_ptr(), q1.stride(0), q1.stride(1),
+                                     k1.stride(0), k1.stride(1), v1.stride(0), v1.stride(1), wide.stride(0), wide.stride(1),
+                                     cu1.data_ptr(), cu1.data_ptr(), 1, 100, 100, hq, hkv, d, 32, 1 / math.sqrt(d),
+                                     0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bool((wide[..., d:] == 7.0).all())
+    ref1 = oracle.staircase_attn_varlen(q1.cpu(), k1.cpu(), v1.cpu(), cu1.cpu(), 32)
+    assert (wide[..., :d].float().cpu() - ref1).abs().max().item() < TOL
