@@ -535,23 +535,68 @@ def idle_loop():
 
 
 def epilogue():
+    """O = O^T / l as bf16 rows.  The accumulators hold O transposed (a lane has 4 consecutive d of its query per
+    d group): stored from there, a store instruction touches 32 rows with 16 bytes each.  Instead every wavefront
+    turns its 32 x 128 tile of one head around through 8 KB of LDS and writes whole rows: 16 lanes x 16 bytes per
+    row, four rows per instruction, 8 instructions per head (before: 16 of half the width, and they cost a tenth
+    of a launch of 1000-token sequences).  The LDS comes from the slot of tile nt + 1: that tile was loaded ahead
+    of need and landed, for every wavefront, before the barrier of the last iteration; nobody reads it and no
+    load still in flight targets it (those are tiles nt + 2 and nt + 3).  Rows use the K / V swizzle (16-byte
+    chunk c of row r at position c ^ (r % 16)), which keeps the 8-byte writes of a (d tile, group) off each
+    other's banks; the reads are linear."""
+    LN, X, WB, RB, L4, OFFL, C0, RV = (f"v{80 + i}" for i in range(8))
+    WA = [f"v{64 + c}" for c in range(16)]
+    SO = [f"v{88 + m}" for m in range(4)]
+    TMP = [f"v{92 + i}" for i in range(2)]
+    OFFJ = [f"v{94 + i}" for i in range(2)]
+    S_STEP = "s47"
     out = [".Lend_%=:", "s_waitcnt lgkmcnt(0)", "s_nop 15", "s_nop 15"]
-    out += [f"v_cmp_ne_u32_e32 vcc, 0, %[ok]", f"s_and_saveexec_b64 {S_SAVE}, vcc"]
+    out += [f"v_mbcnt_lo_u32_b32 {LN}, -1, 0", f"v_mbcnt_hi_u32_b32 {LN}, -1, {LN}",
+            f"v_and_b32_e32 {X}, 15, {LN}", f"v_lshlrev_b32_e32 {X}, 4, {X}",
+            f"v_and_b32_e32 {TMP[0]}, 31, {LN}", f"v_lshlrev_b32_e32 {TMP[0]}, 8, {TMP[0]}",
+            f"v_lshrrev_b32_e32 {TMP[1]}, 5, {LN}", f"v_lshl_add_u32 {TMP[0]}, {TMP[1]}, 3, {TMP[0]}",
+            f"s_add_u32 {S_TMP}, {S_R1}, %[owave]",
+            f"v_add_u32_e32 {WB}, {S_TMP}, {TMP[0]}",
+            f"v_lshl_add_u32 {RB}, {LN}, 4, {S_TMP}",
+            f"v_lshrrev_b32_e32 {L4}, 4, {LN}",
+            f"v_mul_lo_u32 {OFFL}, {L4}, %[ostb]",
+            f"v_lshlrev_b32_e32 {TMP[0]}, 4, {L4}", f"v_xor_b32_e32 {C0}, {TMP[0]}, {X}",
+            f"v_add_u32_e32 {RV}, %[orow0], {L4}"]
+    for c in range(16):
+        out += [f"v_xor_b32_e32 {WA[c]}, {16 * c}, {X}", f"v_add_u32_e32 {WA[c]}, {WA[c]}, {WB}"]
+    for m in range(4):
+        out += [f"v_xor_b32_e32 {SO[m]}, {64 * m}, {C0}", f"v_add_u32_e32 {SO[m]}, {SO[m]}, {OFFL}"]
     for h in range(2):
+        data = [f"v[{96 + 32 * h + 4 * j}:{96 + 32 * h + 4 * j + 3}]" for j in range(8)]
         # l = this lane's partial sum + that of the lane holding the other keys of the same query
         out += [f"v_accvgpr_read_b32 {T[7]}, {lacc(h, 0)}", "s_nop 1", f"v_mov_b32_e32 {T[6]}, {T[7]}", "s_nop 1",
                 f"v_permlane32_swap_b32_e32 {T[7]}, {T[6]}", "s_nop 1",
                 f"v_add_f32_e32 {T[7]}, {T[7]}, {T[6]}", f"v_rcp_f32_e32 {T[7]}, {T[7]}", "s_nop 0"]
         for dt in range(4):
             for g in range(4):
+                n = 4 * dt + g
+                lo = 160 + 6 * (n % 4)                       # four rotating sets of six temporaries
+                f = [f"v{lo + e}" for e in range(6)]
                 for e in range(4):
-                    out.append(f"v_accvgpr_read_b32 {T[2 + e]}, a{64 * h + 16 * dt + 4 * g + e}")
+                    out.append(f"v_accvgpr_read_b32 {f[2 + e]}, a{64 * h + 16 * dt + 4 * g + e}")
                 for e in range(4):
-                    out.append(f"v_mul_f32_e32 {T[2 + e]}, {T[2 + e]}, {T[7]}")
-                out.append(f"v_cvt_pk_bf16_f32 {T[0]}, {T[2]}, {T[3]}")
-                out.append(f"v_cvt_pk_bf16_f32 {T[1]}, {T[4]}, {T[5]}")
-                out.append(f"global_store_dwordx2 %[o{h}], v[16:17], off offset:{(dt * 32 + 8 * g) * 2}")
-    out += [f"s_mov_b64 exec, {S_SAVE}"]
+                    out.append(f"v_mul_f32_e32 {f[2 + e]}, {f[2 + e]}, {T[7]}")
+                out.append(f"v_cvt_pk_bf16_f32 {f[0]}, {f[2]}, {f[3]}")
+                out.append(f"v_cvt_pk_bf16_f32 {f[1]}, {f[4]}, {f[5]}")
+                out.append(f"ds_write_b64 {WA[n]}, v[{lo}:{lo + 1}]")
+        out.append("s_waitcnt lgkmcnt(0)")
+        for j in range(8):
+            out.append(f"ds_read_b128 {data[j]}, {RB} offset:{1024 * j}")
+        for j in range(8):
+            # rows 4 j + lane / 16 of the wavefront: stored where the row lies inside the sequence
+            out += [f"s_mul_i32 {S_STEP}, %[ostb], {4 * j}",
+                    f"v_add_u32_e32 {TMP[j % 2]}, {4 * j}, {RV}",
+                    f"v_add_u32_e32 {OFFJ[j % 2]}, {S_STEP}, {SO[j % 4]}",
+                    f"v_cmp_gt_u32_e32 vcc, %[olen], {TMP[j % 2]}",
+                    f"s_waitcnt lgkmcnt({7 - j})",
+                    f"s_and_saveexec_b64 {S_SAVE}, vcc",
+                    f"global_store_dwordx4 {OFFJ[j % 2]}, {data[j]}, %[ob{h}] nt",
+                    f"s_mov_b64 exec, {S_SAVE}"]
     return out
 
 
@@ -580,8 +625,10 @@ struct PairCoreArgs {
     int jpl;                         // row of the tile whose chunk this lane loads (first of four, 16 apart)
     unsigned ch;                     // byte offset inside a K / V row of the 16-byte chunk this lane loads
     int mrel, mlim;                  // key mask: key visible iff unsigned(key0 + const + mrel) < mlim
-    __bf16* o0; __bf16* o1;          // output rows of the two heads (+ 4 * half-wave elements)
-    int ok;                          // this lane's query row exists
+    const void* ob0; const void* ob1;  // output of the two heads at the wavefront's first row (which may lie before the sequence)
+    unsigned ostb;                   // bytes between consecutive output rows
+    unsigned owave;                  // LDS byte address of this wavefront's 8 KB share of a slot
+    int orow0, olen;                 // the wavefront's first row relative to the sequence's first token; tokens in the sequence
     const void* kb; const void* vb;  // K / V of this KV head, at the (virtual) row of padded key 0
     unsigned krb, vrb;               // bytes between consecutive K / V rows
     unsigned wrow;                   // LDS byte address of the first row this wavefront loads in slot 0
@@ -604,7 +651,8 @@ def main():
     tail = f'''
         :
         : [ka] "v"(A.ka), [val] "v"(A.val), [vah] "v"(A.vah), [jpl] "v"(A.jpl), [ch] "v"(A.ch),
-          [mrel] "v"(A.mrel), [mlim] "v"(A.mlim), [o0] "v"(A.o0), [o1] "v"(A.o1), [ok] "v"(A.ok),
+          [mrel] "v"(A.mrel), [mlim] "v"(A.mlim),
+          [ob0] "s"(A.ob0), [ob1] "s"(A.ob1), [ostb] "s"(A.ostb), [owave] "s"(A.owave), [orow0] "s"(A.orow0), [olen] "s"(A.olen),
           [kb] "s"(A.kb), [vb] "s"(A.vb), [krb] "s"(A.krb), [vrb] "s"(A.vrb), [wrow] "s"(A.wrow),
           [pad] "s"(A.pad), [lpm1] "s"(A.lpm1), [nt] "s"(A.nt), [whm] "s"(A.whm), [whx] "s"(A.whx),
           {qops}

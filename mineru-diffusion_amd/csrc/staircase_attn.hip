@@ -305,9 +305,12 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.wrow = (unsigned)uniform((int)(lds0 + (unsigned)(4 * wave * kRowBytes)));
     A.mrel = 2 * H - pad;
     A.mlim = limit_of(min(ip, Lp - 1)) - pad;
-    A.o0 = P.o + tok * P.o_st + (int64_t)head0 * P.o_sh + 4 * H;
-    A.o1 = A.o0 + P.o_sh;
-    A.ok = row_ok ? 1 : 0;
+    A.ob0 = uniform((const void*)(P.o + ((int64_t)seq0 + (row_w0 - pad)) * P.o_st + (int64_t)head0 * P.o_sh));
+    A.ob1 = uniform((const void*)(P.o + ((int64_t)seq0 + (row_w0 - pad)) * P.o_st + (int64_t)(head0 + 1) * P.o_sh));
+    A.ostb = (unsigned)uniform((int)(P.o_st * 2));
+    A.owave = (unsigned)uniform((int)(lds0 + (unsigned)(wave * 32 * kRowBytes)));
+    A.orow0 = uniform(row_w0 - pad);
+    A.olen = uniform(L);
     A.kb = uniform((const void*)(P.k + (int64_t)kvh * P.k_sh + ((int64_t)seq0 - pad) * P.k_st));
     A.vb = uniform((const void*)(P.v + (int64_t)kvh * P.v_sh + ((int64_t)seq0 - pad) * P.v_st));
     A.krb = (unsigned)uniform((int)(P.k_st * 2));
@@ -379,7 +382,9 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     // other's (64 x 600 tokens: 0.237 against 0.259 ms, 16 x 300: 0.028 against 0.035; equal at 1100 tokens, and
     // from there on the pair kernel wins: 1.3 x at 8 x 4096).
     const bool narrow = head_dim < kHeadDim;                   // one-head kernel, rows padded with zeros
-    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 640 && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
+    // (its epilogue writes rows of o in 16-byte pieces, through 32-bit byte offsets from the wavefront's first row)
+    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 640 && o_stride_t % 8 == 0 && o_stride_h % 8 == 0 && o_stride_t > 0 &&
+                       o_stride_t * 2 * 128 < ((int64_t)1 << 31) && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
