@@ -44,6 +44,7 @@ struct StaircaseParams {
     int batch, n_row_groups, num_q_heads, num_kv_heads;
     int log2_s;
     int head_dim;                                              // <= 128, a multiple of 16
+    int o_rows16;                                              // rows of o take 16-byte stores (aligned, strides multiples of 8 elements)
     float c;                                                   // scale * log2(e)
 };
 
@@ -204,9 +205,39 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
         __syncthreads();
     }
 
-    // ---- epilogue: O = O^T / l, bf16, 4 consecutive d per store ----
+    // ---- epilogue: O = O^T / l as 16-bit rows ----
+    // The accumulators hold O transposed: a lane owns 4 consecutive d of its query per (d tile, group), and stores made
+    // from there touch 32 rows with 16 bytes each (16 such instructions cost 12-20 % of a launch of sequences of a few
+    // hundred tokens).  Each wavefront therefore turns its 32 x 128 tile around through one of the four K / V tile
+    // buffers (the loop's last barrier has retired them) and writes whole rows: 16 lanes x 16 bytes per row, four rows
+    // per instruction.  LDS operations of a wavefront complete in order, so its reads see all of its writes.
+    const float inv = 1.0f / both_halves_sum(st.l[0]);          // rows outside the sequence: never stored
+    if (P.o_rows16) {
+        char* tile = (wave & 2) ? lds_vbuf[wave & 1] : lds_kbuf[wave & 1];
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                typename Elem16<E>::vec4 out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
+                *reinterpret_cast<typename Elem16<E>::vec4*>(tile + r * kLdsPitch + d_of_reg(dt, 4 * g, H) * 2) = out;
+            }
+        __builtin_amdgcn_wave_barrier();
+        const int chunk16 = lane & 15, sub = lane >> 4;
+        if (!NARROW || chunk16 * 8 < width) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int rho = 4 * j + sub;                    // row of the wavefront's tile
+                const int jp = row_w0 + rho;
+                const u32x4 v = *reinterpret_cast<const u32x4*>(tile + rho * kLdsPitch + chunk16 * 16);
+                if (jp >= pad && jp < Lp)
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(P.o + ((int64_t)seq0 + (jp - pad)) * P.o_st + (int64_t)head * P.o_sh + chunk16 * 8));
+            }
+        }
+        return;
+    }
     if (!row_ok) return;
-    const float inv = 1.0f / both_halves_sum(st.l[0]);
     __bf16* orow = P.o + tok * P.o_st + (int64_t)head * P.o_sh;
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -369,6 +400,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.num_q_heads = num_q_heads;
     P.num_kv_heads = num_kv_heads;
     P.head_dim = head_dim;
+    P.o_rows16 = (o_stride_t % 8 == 0 && o_stride_h % 8 == 0) ? 1 : 0;
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
     // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence

@@ -479,3 +479,13 @@ def test_narrow_heads_prefill_and_decode(dev, d, dtype):
     assert bool((wide[..., d:] == 7.0).all())
     ref1 = oracle.staircase_attn_varlen(q1.cpu(), k1.cpu(), v1.cpu(), cu1.cpu(), 32)
     assert (wide[..., :d].float().cpu() - ref1).abs().max().item() < TOL
+    # rows of o whose stride is a multiple of 4 elements but not of 8 take the 8-byte store path
+    odd = torch.full((100, hq, 132), 7.0, dtype=dtype, device=dev)
+    rc = L.mdx_staircase_attn_varlen(q1.data_ptr(), k1.data_ptr(), v1.data_ptr(), odd.data_ptr(), q1.stride(0), q1.stride(1),
+                                     k1.stride(0), k1.stride(1), v1.stride(0), v1.stride(1), odd.stride(0), odd.stride(1),
+                                     cu1.data_ptr(), cu1.data_ptr(), 1, 100, 100, hq, hkv, d, 32, 1 / math.sqrt(d),
+                                     0 if dtype == torch.bfloat16 else 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bool((odd[..., d:] == 7.0).all())
+    assert torch.equal(odd[..., :d], wide[..., :d])
