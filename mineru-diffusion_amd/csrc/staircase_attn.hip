@@ -411,11 +411,11 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     // (the hand-scheduled pair kernel exists for bf16; fp16 runs the one-head kernel).  Sequences of a few hundred
     // tokens are left to the one-head kernel as well: a pair workgroup owns a whole CU and its fixed cost (set-up,
     // prologue, epilogue: 10 us) is then most of its time, while two one-head workgroups share a CU and hide each
-    // other's (64 x 600 tokens: 0.237 against 0.259 ms, 16 x 300: 0.028 against 0.035; equal at 1100 tokens, and
-    // from there on the pair kernel wins: 1.3 x at 8 x 4096).
+    // other's (one-head against pair, ms: 64 x 300 tokens 0.088 / 0.103, 32 x 500 0.074 / 0.081, 64 x 600 0.222 / 0.216,
+    // 32 x 700 0.130 / 0.128, 32 x 800 0.162 / 0.155, 32 x 1000 0.230 / 0.204, 16 x 2048 0.383 / 0.304).
     const bool narrow = head_dim < kHeadDim;                   // one-head kernel, rows padded with zeros
     // (its epilogue writes rows of o in 16-byte pieces, through 32-bit byte offsets from the wavefront's first row)
-    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 640 && o_stride_t % 8 == 0 && o_stride_h % 8 == 0 && o_stride_t > 0 &&
+    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 560 && o_stride_t % 8 == 0 && o_stride_h % 8 == 0 && o_stride_t > 0 &&
                        o_stride_t * 2 * 128 < ((int64_t)1 << 31) && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);

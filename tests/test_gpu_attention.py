@@ -31,7 +31,7 @@ def _check_prefill(dev, lens, S, hq=16, hkv=8, seed=0, max_seqlen=None):
     ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
     err = (o.float().cpu() - ref).abs().max().item()
     assert err < TOL, f"max-abs {err} for lens={lens} S={S}"
-    if max_seqlen is None and sum(lens) <= 640:
+    if max_seqlen is None and sum(lens) <= 560:
         # sequences this short go to the one-head kernel; a larger (still valid) bound selects the pair kernel for
         # even head ratios, so both kernels see every small case
         o2 = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S, max_seqlen=1024)
