@@ -68,7 +68,22 @@ __device__ __forceinline__ void seq_bounds(const StaircaseParams& P, int b, int&
 // this dense numbering itself (lane b holds sequence b's row-group count, lane r evaluates
 // F(r) = #pairs at level >= r); beyond that the grid is the full (level x sequence) rectangle and
 // absent pairs return at once.  Returns false when there is no such pair.
-__device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j, int lane, int& b, int& rg)
+// Inclusive prefix sum over the 64 lanes of a wavefront (DPP shifts inside rows of 16 lanes, then the
+// two row broadcasts): 6 additions, no LDS traffic.
+__device__ __forceinline__ int wave_prefix_sum(int x)
+{
+    int v = x;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// `hist`: 65 ints of LDS that belong to the calling wavefront alone (unused when there are more than 64 row groups).
+__device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j, int lane, int* hist, int& b, int& rg)
 {
     if (P.batch <= 64) {
         int g = 0;                                             // row groups of sequence `lane`
@@ -78,16 +93,36 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
             if (len > 0) g = ((((len + (1 << P.log2_s) - 1) >> P.log2_s) << P.log2_s) + kRowsPerWg - 1) / kRowsPerWg;
         }
         int level = -1, f_level = 0;
-        for (int base = 0; base < P.n_row_groups; base += 64) {
-            const int r_lane = base + lane;
-            int f = 0;
-            for (int s = 0; s < P.batch; ++s) f += max(0, __builtin_amdgcn_readlane(g, s) - r_lane);
-            const unsigned long long above = __ballot(f > j);  // F decreases with the level: low lanes
-            if (above == 0) break;
+        if (P.n_row_groups <= 64) {
+            // F(r) = sum over sequences of max(0, g - r) for all 64 levels r at once, without a loop over the
+            // sequences (which took 0.9 us of every workgroup's start at 32 sequences, 1.8 at 64): count the
+            // sequences per value of g (LDS atomics of this wavefront only, which complete in order), then
+            // C(r) = #{g > r} and F(r) = C(r) + C(r + 1) + ... are two prefix sums with the levels laid out
+            // backwards over the lanes (lane l = level 63 - l).
+            hist[lane] = 0;
+            if (lane == 0) hist[64] = 0;
+            if (lane < P.batch) atomicAdd(&hist[g], 1);        // g <= n_row_groups <= 64
+            __builtin_amdgcn_wave_barrier();
+            const int c = wave_prefix_sum(hist[64 - lane]);    // C(63 - lane)
+            const int f = wave_prefix_sum(c);                  // F(63 - lane)
+            const unsigned long long above = __ballot(f > j);  // the levels 0 .. n - 1: the high lanes
             const int n = __popcll(above);
-            level = base + n - 1;
-            f_level = __builtin_amdgcn_readlane(f, n - 1);
-            if (n < 64) break;
+            if (n > 0) {
+                level = n - 1;
+                f_level = __builtin_amdgcn_readlane(f, 64 - n);
+            }
+        } else {
+            for (int base = 0; base < P.n_row_groups; base += 64) {
+                const int r_lane = base + lane;
+                int f = 0;
+                for (int s = 0; s < P.batch; ++s) f += max(0, __builtin_amdgcn_readlane(g, s) - r_lane);
+                const unsigned long long above = __ballot(f > j);  // F decreases with the level: low lanes
+                if (above == 0) break;
+                const int n = __popcll(above);
+                level = base + n - 1;
+                f_level = __builtin_amdgcn_readlane(f, n - 1);
+                if (n < 64) break;
+            }
         }
         if (level < 0) return false;                           // past the last pair
         const unsigned long long owners = __ballot(g > level); // sequences that have this row group
@@ -96,6 +131,7 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
         const unsigned long long hit = __ballot(((owners >> lane) & 1ull) != 0 && before == nth);
         b = __ffsll((long long)hit) - 1;
         rg = level;
+        if (b < 0) return false;
     } else {
         b = j % P.batch;
         rg = P.n_row_groups - 1 - j / P.batch;
@@ -111,6 +147,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     const int width = NARROW ? P.head_dim : kHeadDim;
     __shared__ __attribute__((aligned(16))) char lds_kbuf[2][kTileBytes];   // double-buffered K and V tiles
     __shared__ __attribute__((aligned(16))) char lds_vbuf[2][kTileBytes];
+    __shared__ int lds_hist[kThreads / 64][80];                // per wavefront: scratch of the workgroup numbering (no barrier separates it from the first tile store)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
@@ -118,7 +155,7 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
     // ---- workgroup -> (head slot, sequence b, row group rg) ------------------------------------
     const int hslot = blockIdx.x % P.num_q_heads;
     int b, rg;
-    if (!locate_row_group(P, blockIdx.x / P.num_q_heads, lane, b, rg)) return;
+    if (!locate_row_group(P, blockIdx.x / P.num_q_heads, lane, lds_hist[wave], b, rg)) return;
 
     int seq0, L;
     seq_bounds(P, b, seq0, L);
@@ -285,7 +322,8 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     const int item = blockIdx.x;
     const int hslot = item % n_hslots;
     int b, rg;
-    if (!locate_row_group(P, item / n_hslots, lane, b, rg)) return;
+    // (scratch for the numbering: in slot 4, which no K/V load targets before every wavefront has passed the core's first barrier)
+    if (!locate_row_group(P, item / n_hslots, lane, reinterpret_cast<int*>(lds_pair + 4 * (2 * kTileKeys * kRowBytes)) + wave * 80, b, rg)) return;
 
     int seq0, L;
     seq_bounds(P, b, seq0, L);
