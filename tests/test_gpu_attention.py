@@ -489,3 +489,30 @@ def test_narrow_heads_prefill_and_decode(dev, d, dtype):
     torch.cuda.synchronize()
     assert bool((odd[..., d:] == 7.0).all())
     assert torch.equal(odd[..., :d], wide[..., :d])
+
+
+def test_prefill_output_rows_honour_the_strides_of_o(dev):
+    """Both staircase kernels write o as whole 256-byte rows through an LDS transpose; the rows go where the strides of
+    o say, and nothing else is touched: o as a slice of a wider buffer (head stride 160, token stride 16 * 160 + 24),
+    lengths on both sides of the one-head / pair switch, a sequence that ends inside a 128-row group, rows before the
+    first token of a right-aligned first block."""
+    import mdx
+    L = mdx._lib.lib()
+    g = torch.Generator().manual_seed(4242)
+    hq, hkv, d = 16, 8, 128
+    for lens in ([333, 100], [700, 37, 1000]):
+        q, k, v, cu = _packed(g, lens, hq, hkv)
+        N = sum(lens)
+        buf = torch.full((N, hq * 160 + 24), 7.0, dtype=torch.bfloat16, device=dev)
+        o = buf[:, :hq * 160].unflatten(-1, (hq, 160))[..., :d]
+        qd, kd, vd, cud = q.to(dev), k.to(dev), v.to(dev), cu.to(dev)
+        rc = L.mdx_staircase_attn_varlen(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), qd.stride(0), qd.stride(1),
+                                         kd.stride(0), kd.stride(1), vd.stride(0), vd.stride(1), o.stride(0), o.stride(1),
+                                         cud.data_ptr(), cud.data_ptr(), len(lens), max(lens), N, hq, hkv, d, 32, 1 / math.sqrt(d), 0,
+                                         torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
+        assert (o.float().cpu() - ref).abs().max().item() < TOL
+        wide = buf[:, :hq * 160].unflatten(-1, (hq, 160))
+        assert bool((wide[..., d:] == 7.0).all()) and bool((buf[:, hq * 160:] == 7.0).all())
