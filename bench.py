@@ -241,7 +241,13 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, maske
     blocks = new_tokens // S
     assert all(s.num_completion_tokens == new_tokens and len(s.step_map) == new_tokens for s in seqs), "incomplete generation"
     assert not any(cfg.mask_token_id in s.completion_token_ids for s in seqs), "mask token in the output"
-    assert st["decode_passes"] == blocks * (steps_per_block + 1) - 1, f"unexpected pass count {st['decode_passes']}"
+    expected = blocks * (steps_per_block + 1) - 1
+    if gumbel_seed is None:
+        assert st["decode_passes"] == expected, f"unexpected pass count {st['decode_passes']}"
+    else:
+        # a sampled draw can be the mask token itself (1 in 151 936 per draw on these logits): the position then stays
+        # masked for another pass, as in the reference (sampler.py:32 looks at the tokens, not at what was committed)
+        assert expected <= st["decode_passes"] <= expected + blocks, f"unexpected pass count {st['decode_passes']}"
     out = dict(tokens_per_s=round(done / dt, 1), seconds=round(dt, 3), committed_tokens=done, batch=batch,
                prefill_passes=st["prefill_passes"], decode_passes=st["decode_passes"],
                prefill_s=round(st["prefill_s"], 3), decode_s=round(st["decode_s"], 3),

@@ -326,52 +326,65 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         __syncthreads();
     }
 
-    // ---- merge the KW key-slice states of each head (tree through LDS) ----------------------
+    // ---- merge the KW key-slice states of each head through LDS ---------------------------------
+    // Every slice leaves its state in LDS (register quads as 16-byte lanes: 16 stores of 1 KB per wavefront); after one
+    // barrier slice kw folds the d tiles kw, kw + KW, ... of all KW states -- every slice a quarter (half) of the head,
+    // and every slice stores what it folded.  (A tree of pairwise merges with 4-byte LDS accesses and three barriers,
+    // all output from one wavefront, took 2.7 us of every workgroup's end.)  All slices sum in the same order, so they
+    // agree on the head's m and l bit for bit.
     st.l[0] = both_halves_sum(st.l[0]);          // a state is now (m, l, O) per query
-    // Exchange layout per sending wavefront: O as [4][16][64 lanes] floats, then m, l as [64].
+    // Exchange layout per wavefront: O as [d tile][group][64 lanes][4] floats, then m, l as [64].
     constexpr int kStateFloats = 4 * 16 * 64 + 2 * 64;
-    static_assert(HPW * (KW / 2) * kStateFloats * 4 <= (int)sizeof(lds), "merge buffer exceeds the tile region");
-    float* xch = reinterpret_cast<float*>(&lds[0][0]);
-    auto send = [&](int slot) {
-        float* dst = xch + slot * kStateFloats;
+    static_assert(HPW * KW * kStateFloats * 4 <= (int)sizeof(lds), "merge buffer exceeds the tile region");
+    float* xch = reinterpret_cast<float*>(&lds[0][0]) + (wave / KW) * KW * kStateFloats;   // this head's slots
+    // (the loop's last barrier already separates the tile reads from these writes)
+    {
+        float* dst = xch + kw * kStateFloats;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = st.o[0][t][i];
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<f32x4*>(dst + ((t * 4 + g) * 64 + lane) * 4) =
+                    f32x4{st.o[0][t][4 * g], st.o[0][t][4 * g + 1], st.o[0][t][4 * g + 2], st.o[0][t][4 * g + 3]};
         dst[4 * 16 * 64 + lane] = st.m[0];
         dst[4 * 16 * 64 + 64 + lane] = st.l[0];
-    };
-    auto recv = [&](int slot) {
-        const float* src = xch + slot * kStateFloats;
-        const float m2 = src[4 * 16 * 64 + lane];
-        const float l2 = src[4 * 16 * 64 + 64 + lane];
-        const float M = fmaxf(st.m[0], m2);
-        const float a1 = __builtin_amdgcn_exp2f(st.m[0] - M), a2 = __builtin_amdgcn_exp2f(m2 - M);
-        st.l[0] = st.l[0] * a1 + l2 * a2;
-        st.m[0] = M;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                st.o[0][t][i] = st.o[0][t][i] * a1 + src[(t * 16 + i) * 64 + lane] * a2;
-    };
-    // (the loop's last barrier already separates the tile reads from these writes)
-#pragma unroll
-    for (int stride = KW / 2; stride >= 1; stride >>= 1) {
-        if (kw >= stride && kw < 2 * stride) send((wave / KW) * stride + (kw - stride));
-        __syncthreads();
-        if (kw < stride) recv((wave / KW) * stride + kw);
-        if (stride > 1) __syncthreads();
     }
-    const bool writer = kw == 0 && row_ok;
+    __syncthreads();
+    {
+        float w[KW];                                // weights of the KW states: 2^(m_s - M)
+        float M = kMinusBig;
+#pragma unroll
+        for (int s = 0; s < KW; ++s) { w[s] = xch[s * kStateFloats + 4 * 16 * 64 + lane]; M = fmaxf(M, w[s]); }
+        float l = 0.f;
+#pragma unroll
+        for (int s = 0; s < KW; ++s) {
+            w[s] = __builtin_amdgcn_exp2f(w[s] - M);
+            l += xch[s * kStateFloats + 4 * 16 * 64 + 64 + lane] * w[s];
+        }
+        st.m[0] = M;
+        st.l[0] = l;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            if (t % KW != kw) continue;             // (uniform per wavefront)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KW; ++s)
+                    acc += *reinterpret_cast<const f32x4*>(xch + s * kStateFloats + ((t * 4 + g) * 64 + lane) * 4) * w[s];
+                st.o[0][t][4 * g] = acc.x; st.o[0][t][4 * g + 1] = acc.y; st.o[0][t][4 * g + 2] = acc.z; st.o[0][t][4 * g + 3] = acc.w;
+            }
+        }
+    }
 
-    // ---- output ---------------------------------------------------------------
+    // ---- output: slice kw holds, and stores, the d tiles kw, kw + KW, ... of its head ----------------
     if (n_valid_splits == 1) {
-        if (!writer) return;
+        if (!row_ok) return;
         const float inv = st.l[0] > 0.f ? 1.0f / st.l[0] : 0.f;   // no valid key at all: zeros
         __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)r * P.o_ss + (int64_t)head * P.o_sh;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 4; ++dt) {
+            if (dt % KW != kw) continue;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 typename Elem16<E>::vec4 out;
@@ -379,20 +392,23 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
                 for (int e = 0; e < 4; ++e) out[e] = (E)(st.o[0][dt][4 * g + e] * inv);
                 if (d_of_reg(dt, 4 * g, H) < P.head_dim) *reinterpret_cast<typename Elem16<E>::vec4*>(orow + d_of_reg(dt, 4 * g, H)) = out;
             }
+        }
         return;
     }
-    if (writer) {
+    if (row_ok) {
         const int64_t slot = ((int64_t)b * P.num_q_heads + head) * P.nsplit + split;
         float* po = P.part_o + (slot * kMaxSq + r) * kHeadDim;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 4; ++dt) {
+            if (dt % KW != kw) continue;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const f32x4 out = {st.o[0][dt][4 * g], st.o[0][dt][4 * g + 1], st.o[0][dt][4 * g + 2], st.o[0][dt][4 * g + 3]};
                 if (P.arrive) store_agent(po + d_of_reg(dt, 4 * g, H), out);
                 else *reinterpret_cast<f32x4*>(po + d_of_reg(dt, 4 * g, H)) = out;
             }
-        if (H == 0) {
+        }
+        if (kw == 0 && H == 0) {
             float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + r;
             if (P.arrive) {
                 __hip_atomic_store(ml, st.m[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
