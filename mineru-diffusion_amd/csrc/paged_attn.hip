@@ -39,10 +39,17 @@ using namespace mdx_attn;
 constexpr int kMaxSq = 32;
 constexpr int kChunkAlign = 256;   // split boundaries are multiples of this many keys
 
+// Sum over the 64 lanes: DPP shifts inside the rows of 16 lanes, the two row broadcasts, the total from lane 63
+// (six additions, no LDS traffic: the butterfly of cross-lane LDS permutes it replaces sat in every workgroup's start).
 __device__ __forceinline__ int wave_sum(int x) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o);
-    return __builtin_amdgcn_readfirstlane(x);      // the same in every lane: say so to the compiler
+    int v = x;
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // Partials that another workgroup of the same launch reads (single-launch merge) travel with
@@ -181,9 +188,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
 
     // ---- workgroup -> (sequence b, split) ------------------------------------------------------
     int b, split, span = P.chunk;
+    int ctx_all = 0;                                // (up to 64 sequences) the clipped length of sequence `lane`
     if (P.bs <= 64) {
         // lengths beyond the page table name keys that do not exist: clipped here and below
         const int ctx_l = lane < P.bs ? min(max(0, P.context_lens[lane]), P.max_pages * P.page_size) : 0;
+        ctx_all = ctx_l;
         if (P.span_out) {
             // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
             // nothing to combine) -- unless one of them is much longer than the rest and would keep
@@ -219,7 +228,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         b = blockIdx.y / P.nsplit;
         split = blockIdx.y % P.nsplit;
     }
-    const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
+    const int ctx = P.bs <= 64 ? __builtin_amdgcn_readlane(ctx_all, b)       // lane b read it above: no second trip to memory
+                               : min(P.context_lens[b], P.max_pages * P.page_size);
     const int n_valid_splits = (ctx + span - 1) / span;
     if (ctx <= 0) {
         // graph-padding row: defined output (zeros), written by its split 0
