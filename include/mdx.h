@@ -69,7 +69,9 @@ int mdx_store_kvcache(const void* key, const void* value,
  * q,o [total_tokens, Hq, d]; k,v [total_tokens, Hkv, d]; the innermost stride
  * is 1, token and head strides are given in elements (so the strided views of
  * a fused QKV projection are read in place; the reference copies them,
- * :182).  cu_seqlens_q / cu_seqlens_k [batch+1] int32 device arrays; the
+ * :182).  q, k, v, o 16-byte aligned; strides of q, k, v multiples of 8
+ * elements, those of o multiples of 4 (multiples of 8 let the kernels write
+ * whole 256-byte rows of o, the faster form).  cu_seqlens_q / cu_seqlens_k [batch+1] int32 device arrays; the
  * kernel is a self-attention and reads the sequence bounds from cu_seqlens_k,
  * like the reference (:48-50); both must describe the same sequences.
  * Blocks of staircase_size tokens (1,2,..,128) are right-aligned in every
