@@ -10,9 +10,11 @@
 // and a 16-bit logit has only 65 536 possible values, so that value is found by counting: one pass
 // histograms the high byte of an order-preserving key (element count and probability mass per bin),
 // the bin where the running count / mass crosses the target is found, and a second pass histograms the
-// low byte inside that bin.  Two passes per filter (top-p a third before them, for the row maximum
-// that its softmax terms are relative to) and one pass that writes the filtered copy, all over a row
-// that the first pass has pulled into the cache hierarchy; one workgroup per row.
+// low byte inside that bin.  Two passes per filter (top-p needs the row maximum that its softmax terms are
+// relative to: the first top-k pass finds it on the way, a top-p without top-k takes a pass for it) and one
+// pass that writes the filtered copy; one workgroup per row.  Every pass reads the row from memory again (the
+// rows in flight exceed the L2), and with two workgroups per CU that traffic and the LDS atomics of the
+// counting cost about the same: holding the row in registers (one workgroup per CU) measured slower.
 //
 // Where the reference's sort leaves the order of equal values open, all elements equal to the crossing
 // value are kept.  The probability masses are fp32 terms summed in fixed point, so the result does not
@@ -88,9 +90,12 @@ struct Shared {
 // first exceeds top_p of the total : the key of the k-th largest.  Returns floor_key when the
 // target is never reached (k at or beyond the number of such elements).  Masses are softmax terms
 // relative to the row maximum m, exp2((x - m) * c) <= 1.
-template <typename T, bool MASS>
+// TRACK_MAX: the first pass also leaves the key of the row's largest element in sh.max_key (which the caller has
+// cleared), so that a top-p selection that follows needs no pass of its own for it.
+template <typename T, bool MASS, bool TRACK_MAX = false>
 __device__ uint32_t select_key(const RowView& row, Shared& sh, uint32_t floor_key, int k, float top_p, float c, float m) {
     const int tid = threadIdx.x, slot = tid % kSlots;
+    uint32_t mk = 0;
     auto clear_slots = [&]() {
         for (int i = tid; i < 256 * kSlots; i += kFilterThreads) { sh.cnt_slots[i] = 0; if (MASS) sh.mass_slots[i] = 0ull; }
         __syncthreads();
@@ -113,11 +118,17 @@ __device__ uint32_t select_key(const RowView& row, Shared& sh, uint32_t floor_ke
     clear_slots();
     scan_row(row, tid, [&](uint32_t b) {
         const uint32_t key = key_of(b);
+        if (TRACK_MAX) mk = key > mk ? key : mk;
         if (key < floor_key) return;
         const int at = (int)(key >> 8) * kSlots + slot;
         atomicAdd(&sh.cnt_slots[at], 1);
         if (MASS) atomicAdd(&sh.mass_slots[at], (unsigned long long)(__builtin_amdgcn_exp2f((Bits16<T>::value(b) - m) * c) * kMassScale));
     });
+    if (TRACK_MAX) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) { const uint32_t o = __shfl_xor(mk, off); mk = o > mk ? o : mk; }
+        if ((tid & 63) == 0) atomicMax(&sh.max_key, mk);
+    }
     sum_slots();
     if (tid == 0) {
         float target = 0.f;
@@ -196,16 +207,19 @@ __global__ __launch_bounds__(kFilterThreads) void logit_filter_kernel(
     const float c = kLog2e / T_;
 
     uint32_t floor_key = 0;
-    if (top_k > 0 && top_k < vocab) floor_key = select_key<T, false>(row, sh, floor_key, top_k, 1.f, c, 0.f);
+    if (tid == 0) sh.max_key = 0;
+    __syncthreads();
+    const bool with_k = top_k > 0 && top_k < vocab;
+    if (with_k) floor_key = select_key<T, false, true>(row, sh, floor_key, top_k, 1.f, c, 0.f);   // also finds the row maximum
     if (top_p < 1.0f) {
-        if (tid == 0) sh.max_key = 0;
-        __syncthreads();
-        uint32_t mk = 0;
-        scan_row(row, tid, [&](uint32_t b) { const uint32_t key = key_of(b); mk = key > mk ? key : mk; });
+        if (!with_k) {
+            uint32_t mk = 0;
+            scan_row(row, tid, [&](uint32_t b) { const uint32_t key = key_of(b); mk = key > mk ? key : mk; });
 #pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) { const uint32_t o = __shfl_xor(mk, off); mk = o > mk ? o : mk; }
-        if ((tid & 63) == 0) atomicMax(&sh.max_key, mk);
-        __syncthreads();
+            for (int off = 32; off >= 1; off >>= 1) { const uint32_t o = __shfl_xor(mk, off); mk = o > mk ? o : mk; }
+            if ((tid & 63) == 0) atomicMax(&sh.max_key, mk);
+            __syncthreads();
+        }
         // a row whose largest element is not finite has no softmax to take a share of: left as it is
         const float m = Bits16<T>::value(bits_of(sh.max_key));
         if (m > -INFINITY && m < INFINITY)
