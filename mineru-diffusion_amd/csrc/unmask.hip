@@ -173,6 +173,7 @@ __device__ __forceinline__ U4 philox4x32_10(U4 c, uint32_t k0, uint32_t k1) {
 // exponential.  With t = log2 u: -ln(-ln u) = -ln 2 * log2(-t) - ln(ln 2).  The largest noise values, the ones
 // that decide an argmax, come from u next to 1, where t is tiny: the hardware logarithm keeps its relative
 // accuracy there (over all 2^23 values of u the result is within 2e-6 of the fp64 one).
+constexpr float kGumbelMax = 17.0f;      // above every value of gumbel_of (16.64 at u = 1 - 2^-24)
 __device__ __forceinline__ float gumbel_of(uint32_t bits) {
     const float u = __builtin_fmaf((float)(bits >> 9), 1.1920928955078125e-07f, 5.9604644775390625e-08f);   // (k + 1/2) * 2^-23
     const float t = __builtin_amdgcn_logf(u);
@@ -233,6 +234,11 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
 
     Partial p;
     p.m = kNegBig; p.s = 0.f; p.idx = kNoIndex; p.pick = kNegBig; p.pick_x = 0.f; p.pick_idx = kNoIndex;
+    __shared__ float lead_seen;              // mode 2: the best noisy logit any wavefront of the workgroup has published
+    if (NOISE == 2) {
+        if (tid == 0) lead_seen = kNegBig;
+        __syncthreads();
+    }
 
     // Softmax over 16-byte chunks (modes 0 and 2).  Per lane: running max m, h = -(m * c) rounded to fp32,
     // and s = sum of exp2(x * c + h), each exponent one FMA (x * c + h is rounded once, so the term of x == m is exp2(lo) with
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
     // 2^-24 |m c|, into every term (1e-3 at logits of thousands).
     float m = kNegBig, s = 0.f, h = 0.f;
     int first_at = -1;           // element (counted from the first aligned chunk) that first held m
-    auto take_values = [&](const float (&x)[EPC], int64_t chunk) {
+    auto take_values = [&](const float (&x)[EPC], int64_t chunk) -> float {     // returns the chunk's largest element
         float cm = x[EPC - 1];
 #pragma unroll
         for (int i = 0; i + 2 < EPC; i += 2) cm = max3(cm, x[i], x[i + 1]);
@@ -263,6 +269,7 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
 #pragma unroll
         for (int i = 1; i < EPC; ++i) acc += fast_exp2(__builtin_fmaf(x[i], c, h));
         s += acc;
+        return cm;
     };
     auto lane_softmax_done = [&]() {
         if (m > kNegBig) s *= fast_exp2(-__builtin_fmaf(m, c, h));   // to the base of m itself (a lane that saw no finite element keeps s == 0)
@@ -323,7 +330,8 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
         const bool noise_lines_up = NOISE == 1 && (reinterpret_cast<uintptr_t>(np + lead) & 15) == 0;
         const bool unit_T = T_ == 1.0f;
         float best = kNegBig, best_x = 0.f;
-        int best_idx = kNoIndex;
+        float seen = kNegBig;            // mode 2: what this wavefront knows of the workgroup's best noisy logit (same in all lanes)
+        int best_idx = kNoIndex, since_look = 0;
         auto offer = [&](float x, int index, float g) {
             const float v = (unit_T ? x : x / T_) + g;
             if (v > best || (v == best && index < best_idx)) { best = v; best_x = x; best_idx = index; }
@@ -332,8 +340,21 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
         for (int64_t ch = cbeg + tid; ch < cend; ch += kThreads) {
             float x[EPC];
             Elem<T>::unpack(__builtin_nontemporal_load(cp + ch), x);
-            take_values(x, ch);
+            const float cmx = take_values(x, ch);
             const int c0 = (int)(lead + ch * EPC);
+            // No draw of the generator exceeds kGumbelMax, and rounding is monotonic: an element of this chunk can
+            // take (or tie) the row's lead only if (largest element) / T + kGumbelMax reaches the best noisy logit
+            // that anybody in the workgroup has found so far (lead_seen: published by the wavefronts as they go; an
+            // old value only makes the test more cautious).  Where that holds in no lane of the wavefront the
+            // chunk's noise is not drawn -- every chunk of -inf that a top-k / top-p filter left behind, and the
+            // bulk of a peaked row; what is skipped could not have been picked.  (A noise tensor may hold
+            // anything: mode 1 reads all of it.)
+            if (NOISE == 2) {
+                if ((++since_look & 7) == 0)           // the others' news every eighth chunk: an LDS read per chunk would cost what it saves
+                    seen = fmaxf(seen, __hip_atomic_load(&lead_seen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+                const bool may_lead = (unit_T ? cmx : cmx / T_) + kGumbelMax >= fmaxf(best, seen);
+                if (__builtin_amdgcn_ballot_w64(may_lead) == 0) continue;
+            }
             if (NOISE == 1) {
                 float g[EPC];
                 if (noise_lines_up) {
@@ -361,6 +382,16 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
             } else {
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) offer(x[i], c0 + i, rn.at(c0 + i));
+            }
+            if (NOISE == 2) {
+                // the wavefront's best so far, to everybody (only when it has grown: few chunks of a row raise it)
+                if (__builtin_amdgcn_ballot_w64(best > seen) != 0) {
+                    float wb = best;
+#pragma unroll
+                    for (int off = 32; off >= 1; off >>= 1) wb = fmaxf(wb, __shfl_xor(wb, off));
+                    seen = fmaxf(seen, wb);
+                    if ((tid & (mdx::kWave - 1)) == 0) __hip_atomic_fetch_max(&lead_seen, wb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
             }
         }
         lane_softmax_done();

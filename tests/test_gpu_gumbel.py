@@ -81,6 +81,38 @@ def test_seeded_sampling_equals_sampling_with_the_noise_tensor(dev, dtype, bs, S
         assert not torch.equal(x0, x0b)                                     # another offset, another draw
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_seeded_sampling_of_peaked_rows_skips_only_what_cannot_win(dev, dtype):
+    """The seeded kernel leaves the generator alone for chunks none of whose elements could take the lead (largest
+    element + the largest possible draw below the lane's best so far): rows with a few candidates far above a bulk 20
+    to 60 below them, with stretches of -inf, with the candidates early, late or clustered, at several temperatures
+    -- the picks must be those of the kernel that reads the same noise from a tensor and skips nothing."""
+    import mdx
+    g = torch.Generator().manual_seed(77)
+    bs, S, V = 3, 16, 50000
+    logits = torch.randn(bs, S, V, generator=g) * 2 - 40
+    for b in range(bs):
+        for r in range(S):
+            n = int(torch.randint(1, 40, (1,), generator=g))
+            where = torch.randint(0, V, (n,), generator=g) if r % 3 else torch.arange(V - n, V) if r % 2 else torch.arange(n)
+            logits[b, r, where] = torch.randn(n, generator=g) * 3 + (0 if r % 4 else 15)
+            if r % 5 == 0:
+                lo = int(torch.randint(0, V - 9000, (1,), generator=g))
+                keep = logits[b, r, where].clone()
+                logits[b, r, lo:lo + 9000] = float("-inf")
+                logits[b, r, where] = keep
+    logits = logits.to(dtype).to(dev)
+    temps = torch.tensor([0.5, 1.0, 2.5], device=dev)
+    for offset in range(3):
+        x0, p = mdx.confidence_argmax(logits, temps, seed=11, offset=offset)
+        noise = mdx.gumbel_noise(bs * S, V, 11, offset, device=dev)
+        x0n, pn = mdx.confidence_argmax(logits, temps, noise=noise.view(bs, S, V))
+        torch.cuda.synchronize()
+        assert torch.equal(x0, x0n)
+        torch.testing.assert_close(p, pn, rtol=3e-6, atol=0)
+    assert len(set(x0.flatten().tolist())) > 10
+
+
 def test_seeded_unmask_step_equals_the_step_with_the_noise_tensor(dev):
     import mdx
     g = torch.Generator().manual_seed(3)
