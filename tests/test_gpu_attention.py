@@ -500,11 +500,11 @@ def test_prefill_output_rows_honour_the_strides_of_o(dev):
     L = mdx._lib.lib()
     g = torch.Generator().manual_seed(4242)
     hq, hkv, d = 16, 8, 128
-    for lens in ([333, 100], [700, 37, 1000]):
+    for lens, hs in (([333, 100], 160), ([700, 37, 1000], 160), ([700, 37, 1000], 132)):   # 132: 8-byte rows only, one-head kernel
         q, k, v, cu = _packed(g, lens, hq, hkv)
         N = sum(lens)
-        buf = torch.full((N, hq * 160 + 24), 7.0, dtype=torch.bfloat16, device=dev)
-        o = buf[:, :hq * 160].unflatten(-1, (hq, 160))[..., :d]
+        buf = torch.full((N, hq * hs + 24), 7.0, dtype=torch.bfloat16, device=dev)
+        o = buf[:, :hq * hs].unflatten(-1, (hq, hs))[..., :d]
         qd, kd, vd, cud = q.to(dev), k.to(dev), v.to(dev), cu.to(dev)
         rc = L.mdx_staircase_attn_varlen(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), qd.stride(0), qd.stride(1),
                                          kd.stride(0), kd.stride(1), vd.stride(0), vd.stride(1), o.stride(0), o.stride(1),
@@ -514,5 +514,5 @@ def test_prefill_output_rows_honour_the_strides_of_o(dev):
         torch.cuda.synchronize()
         ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
         assert (o.float().cpu() - ref).abs().max().item() < TOL
-        wide = buf[:, :hq * 160].unflatten(-1, (hq, 160))
-        assert bool((wide[..., d:] == 7.0).all()) and bool((buf[:, hq * 160:] == 7.0).all())
+        wide = buf[:, :hq * hs].unflatten(-1, (hq, hs))
+        assert bool((wide[..., d:] == 7.0).all()) and bool((buf[:, hq * hs:] == 7.0).all())
