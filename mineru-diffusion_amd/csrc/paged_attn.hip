@@ -92,12 +92,16 @@ struct PagedParams {
 };
 
 // Merges the nv split partials of query s of (sequence b, head hq); the caller's 8 threads c = 0..7
-// of a query take 16 consecutive d values each.
-template <typename E, bool AGENT>
-__device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, int nv)
+// of a query take 16 consecutive d values each.  nv comes from `count()`, which is asked only after the
+// loads of the first four slots are on their way: where those slots lie does not depend on it (slots
+// beyond nv hold leftovers and are masked out), so a caller whose split count is still in flight from
+// memory overlaps that latency with the partials'.
+template <typename E, bool AGENT, typename Count>
+__device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, Count count)
 {
     if (c * 16 >= P.head_dim) return;
     const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
+    int nv = P.nsplit;                         // until count() is in: every slot that exists
     float M = kMinusBig, Lsum = 0.f;
     float acc[16];
 #pragma unroll
@@ -107,7 +111,7 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
         f32x4 po[4][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int64_t slot = slot0 + min(i0 + i, nv - 1);
+            const int64_t slot = slot0 + min(i0 + i, P.nsplit - 1);
             const float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + s;
             const float* src = P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16;
             if (AGENT) {
@@ -129,6 +133,10 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(po[i][k]) :: "memory");
+        }
+        if (i0 == 0) {
+            nv = count();
+            if (nv <= 1) return;               // written directly by the attention kernel
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) m[i] = i0 + i < nv ? m[i] : kMinusBig;
@@ -445,7 +453,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     if (!i_am_last) return;
     for (int e = tid; e < HPW * 256; e += kThreads) {
         const int s = (e & 255) >> 3;
-        if (s < P.sq) combine_query<E, true>(P, b, hg * HPW + (e >> 8), s, e & 7, n_valid_splits);
+        if (s < P.sq) combine_query<E, true>(P, b, hg * HPW + (e >> 8), s, e & 7, [&]() { return n_valid_splits; });
     }
     if (tid == 0) __hip_atomic_store(counter, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
@@ -459,13 +467,13 @@ template <typename E>
 __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
     const int hq = blockIdx.x % P.num_q_heads, b = blockIdx.x / P.num_q_heads;
-    const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
-    const int span = P.span_out ? (int)*P.span_out : P.chunk; // the attention kernel's choice
-    const int nv = (ctx + span - 1) / span;
-    if (nv <= 1) return;                                   // written directly by the attention kernel
     const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
     if (s >= P.sq) return;
-    combine_query<E, false>(P, b, hq, s, c, nv);
+    combine_query<E, false>(P, b, hq, s, c, [&]() {
+        const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
+        const int span = P.span_out ? (int)*P.span_out : P.chunk;     // the attention kernel's choice
+        return (ctx + span - 1) / span;
+    });
 }
 
 // Keys per split.  Measured over batches of 4 to 64 sequences and contexts of 300 to 8000 keys, the
