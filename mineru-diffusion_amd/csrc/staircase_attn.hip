@@ -26,6 +26,7 @@
 // XCD L2 when there are 8 KV heads).
 #include "mdx_common.h"
 #include "attn_tile.h"
+#include <atomic>
 
 namespace {
 
@@ -459,9 +460,17 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
     if (pairs) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(staircase_pair_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
-        MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
+        // the kernel's LDS limit is raised once per device (the attribute belongs to the device's copy of the kernel)
+        static std::atomic<bool> lds_limit_raised[64];
+        int device = 0;
+        hipError_t e = hipGetDevice(&device);
+        MDX_REQUIRE(e == hipSuccess && device >= 0 && device < 64, MDX_ELAUNCH, "staircase_attn: no current device (%s)", hipGetErrorString(e));
+        if (!lds_limit_raised[device].load(std::memory_order_acquire)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(staircase_pair_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
+            MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
+            lds_limit_raised[device].store(true, std::memory_order_release);
+        }
         staircase_pair_kernel<<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
     } else if (dtype == MDX_F16) {
         if (narrow) staircase_attn_kernel<_Float16, true><<<(unsigned)grid, kThreads, 0, stream>>>(P);
