@@ -86,8 +86,8 @@ int mdx_store_kvcache(const void* key, const void* value,
  * up to 128 (the reference kernel takes BLOCK_DMODEL = head_dim, :183; widths
  * below 128 run as 128 with zero padding, in the one-head-per-wavefront
  * kernel, and only d columns of o are written), dtype MDX_BF16 or MDX_F16
- * (the reference kernel takes q's dtype, :179-197; fp16 runs the one-head
- * kernel too, about 0.8 x the bf16 rate).
+ * (the reference kernel takes q's dtype, :179-197; both run the same
+ * kernels, fp16 within a few percent of bf16).
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                               int64_t q_stride_t, int64_t q_stride_h,

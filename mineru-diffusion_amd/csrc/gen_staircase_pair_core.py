@@ -40,6 +40,17 @@ Physical registers (all clobbered; the compiler keeps v0..v15 and a128..a191, a2
 """
 import sys
 
+# Element type of q / k / v / o: "bf16" (default) or "f16" (python gen_staircase_pair_core.py f16).  The two cores differ
+# in the MFMA mnemonics, the bit pattern of 1.0 and the float -> element conversions: probabilities are packed by one
+# instruction either way (round to nearest even for bf16; fp16 has only the round-toward-zero pack, whose bias the
+# row sums share, since they are taken from the packed values), the output is rounded to nearest even in both.
+DT = sys.argv[1] if len(sys.argv) > 1 else "bf16"
+assert DT in ("bf16", "f16")
+MFMA = f"v_mfma_f32_32x32x16_{DT}"
+MFMA_SUM = f"v_mfma_f32_4x4x4_16b_{DT}"
+ONE_PAIR = "0x3f803f80" if DT == "bf16" else "0x3c003c00"
+CVT_P = "v_cvt_pk_bf16_f32" if DT == "bf16" else "v_cvt_pkrtz_f16_f32"
+
 ROW = 256
 K_BYTES = 64 * ROW                 # 16384: K part of a slot; V part follows
 SLOT = 2 * K_BYTES
@@ -136,15 +147,17 @@ def softmax_plan(cb, masked):
         r = sreg(cb, h, u, 8 * t + j)
         ops = []
         if masked:
-            ops += [f"v_add_u32_e32 {T[j % 4]}, {key_const(u, 8 * t + j)}, {MREL}",
-                    f"v_cmp_lt_u32_e32 vcc, {T[j % 4]}, %[mlim]",
+            # temporaries T[4..7]: the row maximum of the other tile accumulates in T[0..3] during items 18..25,
+            # which overlap the last of these (items 16..19)
+            ops += [f"v_add_u32_e32 {T[4 + j % 4]}, {key_const(u, 8 * t + j)}, {MREL}",
+                    f"v_cmp_lt_u32_e32 vcc, {T[4 + j % 4]}, %[mlim]",
                     f"v_cndmask_b32_e32 v{r}, {NEG_INF}, v{r}, vcc"]
         return ops + [f"v_exp_f32_e32 v{r}, v{r}"]
 
     def cvt_op(c, j):
         h, u, t = chunks[c]
         base = sreg(cb, h, u, 8 * t)
-        return f"v_cvt_pk_bf16_f32 v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}"
+        return f"{CVT_P} v{base + j}, v{base + 2 * j}, v{base + 2 * j + 1}"
 
     last_exp_item = {}
     for e in range(48):                               # chunks 0..5: three values per QK item
@@ -292,7 +305,7 @@ def qk_items(nb):
         u, ks = n & 1, n >> 1
         rd = lambda frag, u=u, ks=ks: [f"ds_read_b128 {frag[0]}, {KA[ks]}" + (f" offset:{u * 32 * ROW}" if u else "")]
         mf = lambda frag, u=u, ks=ks: [
-            f"v_mfma_f32_32x32x16_bf16 {stup(nb, h, u)}, {frag[0]}, %[q{h}{ks}], {negm(h) if ks == 0 else stup(nb, h, u)}"
+            f"{MFMA} {stup(nb, h, u)}, {frag[0]}, %[q{h}{ks}], {negm(h) if ks == 0 else stup(nb, h, u)}"
             for h in range(2)]
         items.append((rd, mf))
     return items
@@ -308,8 +321,8 @@ def pv_items(cb):
         rd = lambda frag, dt=dt, sfx=sfx: [f"ds_read_b64_tr_b16 {frag[1]}, {VA[0][dt]}{sfx}",
                                            f"ds_read_b64_tr_b16 {frag[2]}, {VA[1][dt]}{sfx}"]
         mf = lambda frag, u=u, t=t, dt=dt: [
-            f"v_mfma_f32_32x32x16_bf16 {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)] + (
-            [f"v_mfma_f32_4x4x4_16b_bf16 {lacc(h)}, {ONES}, {phalf(cb, h, u, t, half)}, {lacc(h)}"
+            f"{MFMA} {otup(h, dt)}, {frag[0]}, {ptup(cb, h, u, t)}, {otup(h, dt)}" for h in range(2)] + (
+            [f"{MFMA_SUM} {lacc(h)}, {ONES}, {phalf(cb, h, u, t, half)}, {lacc(h)}"
              for half in range(2) for h in range(2)] if dt == 1 else [])
         items.append((rd, mf))
     return items
@@ -373,7 +386,7 @@ def prologue():
             out += first + ["s_nop 0"] + last
     out += load_offset_ops()
     for i in range(2):
-        out.append(f"v_mov_b32_e32 v{52 + i}, 0x3f803f80")
+        out.append(f"v_mov_b32_e32 v{52 + i}, {ONE_PAIR}")
     for i in list(range(128)) + [192 + 16 * h + j for h in range(2) for j in range(L_REGS)]:
         out.append(f"v_accvgpr_write_b32 a{i}, 0")
     out += [f"s_waitcnt vmcnt({2 * DMA_PER_TILE})", "s_barrier"]      # tiles 0 and 1 have landed
@@ -581,8 +594,14 @@ def epilogue():
                     out.append(f"v_accvgpr_read_b32 {f[2 + e]}, a{64 * h + 16 * dt + 4 * g + e}")
                 for e in range(4):
                     out.append(f"v_mul_f32_e32 {f[2 + e]}, {f[2 + e]}, {T[7]}")
-                out.append(f"v_cvt_pk_bf16_f32 {f[0]}, {f[2]}, {f[3]}")
-                out.append(f"v_cvt_pk_bf16_f32 {f[1]}, {f[4]}, {f[5]}")
+                if DT == "bf16":
+                    out.append(f"v_cvt_pk_bf16_f32 {f[0]}, {f[2]}, {f[3]}")
+                    out.append(f"v_cvt_pk_bf16_f32 {f[1]}, {f[4]}, {f[5]}")
+                else:
+                    for e in range(4):
+                        out.append(f"v_cvt_f16_f32_e32 {f[2 + e]}, {f[2 + e]}")
+                    out.append(f"v_pack_b32_f16 {f[0]}, {f[2]}, {f[3]}")
+                    out.append(f"v_pack_b32_f16 {f[1]}, {f[4]}, {f[5]}")
                 out.append(f"ds_write_b64 {WA[n]}, v[{lo}:{lo + 1}]")
         out.append("s_waitcnt lgkmcnt(0)")
         for j in range(8):
@@ -619,7 +638,13 @@ HEADER = '''// GENERATED by gen_staircase_pair_core.py -- do not edit; change th
 // docstring for the schedule, the LDS layout and the register map).  Everything between the loads
 // of Q and the stores of O happens inside this one asm statement; the physical registers it uses
 // are declared as clobbers, the operands are read-only.
-struct PairCoreArgs {
+@@STRUCT@@__device__ __forceinline__ void @@NAME@@(const PairCoreArgs& A, const @@VEC@@ (&q)[2][8])
+{
+    asm volatile(
+'''
+
+
+STRUCT = '''struct PairCoreArgs {
     unsigned ka;                     // per-lane LDS byte address of this lane's K fragment of k-step 0 in slot 0
     unsigned val, vah;               // same for the two rows of the V^T fragment of d tile 0
     int jpl;                         // row of the tile whose chunk this lane loads (first of four, 16 apart)
@@ -635,9 +660,6 @@ struct PairCoreArgs {
     int pad, lpm1, nt, whm, whx;     // first valid padded key, last valid padded key, key tiles, first and last key limit of this wavefront
 };
 
-__device__ __forceinline__ void staircase_pair_core(const PairCoreArgs& A, const bf16x8 (&q)[2][8])
-{
-    asm volatile(
 '''
 
 
@@ -661,7 +683,11 @@ def main():
           {aclob});
 }}
 '''
-    sys.stdout.write(HEADER + text + tail)
+    header = HEADER.replace("@@STRUCT@@", STRUCT if DT == "bf16" else "// (PairCoreArgs: see staircase_pair_core.inc, which is included first)\n\n")
+    header = header.replace("@@NAME@@", "staircase_pair_core" if DT == "bf16" else "staircase_pair_core_f16").replace("@@VEC@@", "bf16x8" if DT == "bf16" else "f16x8")
+    if DT != "bf16":
+        header = header.replace("gen_staircase_pair_core.py --", "gen_staircase_pair_core.py f16 --")
+    sys.stdout.write(header + text + tail)
     sys.stderr.write(f"{len(prog)} instructions\n")
 
 

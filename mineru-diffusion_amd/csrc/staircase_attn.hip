@@ -298,6 +298,9 @@ __global__ __launch_bounds__(kThreads, 2) void staircase_attn_kernel(const Stair
 // wavefronts of a workgroup walk the same number of key tiles (they share the tiles' loads and a
 // barrier per tile); for tiles beyond a wavefront's own last limit it only loads and waits.
 #include "staircase_pair_core.inc"
+#include "staircase_pair_core_f16.inc"      // the same core on fp16 elements (the generator run with "f16")
+__device__ __forceinline__ void pair_core(const PairCoreArgs& A, const bf16x8 (&q)[2][8]) { staircase_pair_core(A, q); }
+__device__ __forceinline__ void pair_core(const PairCoreArgs& A, const f16x8 (&q)[2][8]) { staircase_pair_core_f16(A, q); }
 
 constexpr int kPairSlots = 5;                     // LDS slots of one K tile + one V tile, 256-byte rows
 constexpr int kPairLdsBytes = kPairSlots * 2 * kTileKeys * kRowBytes;
@@ -310,6 +313,7 @@ __device__ __forceinline__ const void* uniform(const void* p) {
     return (const void*)(((uint64_t)hi << 32) | lo);
 }
 
+template <typename E>
 __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const StaircaseParams P)
 {
     extern __shared__ __attribute__((aligned(1024))) char lds_pair[];
@@ -344,14 +348,14 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     const bool row_ok = ip >= pad && ip < Lp;
     const int64_t tok = (int64_t)seq0 + (ip - pad);
     // Q^T fragments, pre-multiplied by scale * log2(e) (the MFMA then yields scores in log2 units)
-    bf16x8 q[2][8];
+    typename Elem16<E>::vec8 q[2][8];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         load_q(q[h], row_ok ? P.q + tok * P.q_st + (int64_t)(head0 + h) * P.q_sh : nullptr, H);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) q[h][ks][j] = (__bf16)((float)q[h][ks][j] * P.c);
+            for (int j = 0; j < 8; ++j) q[h][ks][j] = (E)((float)q[h][ks][j] * P.c);
     }
 
     auto limit_of = [&](int row) { return min(Lp, ((row >> P.log2_s) + 1) << P.log2_s); };
@@ -390,7 +394,7 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
     A.nt = uniform((wg_hi + kTileKeys - 1) / kTileKeys);
     A.whm = uniform(limit_of(min(row_w0, Lp - 1)));
     A.whx = uniform(row_w0 < Lp ? limit_of(min(row_w0 + 31, Lp - 1)) : 0);   // tiles from here on hold nothing this wavefront may see
-    staircase_pair_core(A, q);
+    pair_core(A, q);
 }
 
 }  // namespace
@@ -447,31 +451,33 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
                                         : (int64_t)P.n_row_groups * batch;
     // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
     const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
-    // (the hand-scheduled pair kernel exists for bf16; fp16 runs the one-head kernel).  Sequences of a few hundred
-    // tokens are left to the one-head kernel as well: a pair workgroup owns a whole CU and its fixed cost (set-up,
+    // Sequences of a few hundred tokens are left to the one-head kernel: a pair workgroup owns a whole CU and its fixed cost (set-up,
     // prologue, epilogue: 10 us) is then most of its time, while two one-head workgroups share a CU and hide each
     // other's (one-head against pair, ms: 64 x 300 tokens 0.088 / 0.103, 32 x 500 0.074 / 0.081, 64 x 600 0.222 / 0.216,
     // 32 x 700 0.130 / 0.128, 32 x 800 0.162 / 0.155, 32 x 1000 0.230 / 0.204, 16 x 2048 0.383 / 0.304).
     const bool narrow = head_dim < kHeadDim;                   // one-head kernel, rows padded with zeros
     // (its epilogue writes rows of o in 16-byte pieces, through 32-bit byte offsets from the wavefront's first row)
-    const bool pairs = dtype == MDX_BF16 && !narrow && max_l > 560 && o_stride_t % 8 == 0 && o_stride_h % 8 == 0 && o_stride_t > 0 &&
+    const bool pairs = !narrow && max_l > 560 && o_stride_t % 8 == 0 && o_stride_h % 8 == 0 && o_stride_t > 0 &&
                        o_stride_t * 2 * 128 < ((int64_t)1 << 31) && (num_q_heads / num_kv_heads) % 2 == 0 && k_stride_t > 0 && v_stride_t > 0 &&
                        (max_l + 2 * rows_per_wg) * row_elems * 2 < ((int64_t)1 << 31) && row_elems * 2 < (1 << 24) && max_l + 2 * rows_per_wg < (1 << 24);
     const int64_t grid = n_pairs * (pairs ? num_q_heads / 2 : num_q_heads);
     MDX_REQUIRE(grid < ((int64_t)1 << 31), MDX_EUNSUPPORTED, "staircase_attn: grid too large");
     if (pairs) {
         // the kernel's LDS limit is raised once per device (the attribute belongs to the device's copy of the kernel)
-        static std::atomic<bool> lds_limit_raised[64];
+        static std::atomic<bool> lds_limit_raised[2][64];
         int device = 0;
         hipError_t e = hipGetDevice(&device);
         MDX_REQUIRE(e == hipSuccess && device >= 0 && device < 64, MDX_ELAUNCH, "staircase_attn: no current device (%s)", hipGetErrorString(e));
-        if (!lds_limit_raised[device].load(std::memory_order_acquire)) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void*>(staircase_pair_kernel),
+        const bool half = dtype == MDX_F16;
+        if (!lds_limit_raised[half][device].load(std::memory_order_acquire)) {
+            e = hipFuncSetAttribute(half ? reinterpret_cast<const void*>(staircase_pair_kernel<_Float16>)
+                                         : reinterpret_cast<const void*>(staircase_pair_kernel<__bf16>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
             MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "staircase_attn: cannot reserve %d bytes of LDS (%s)", kPairLdsBytes, hipGetErrorString(e));
-            lds_limit_raised[device].store(true, std::memory_order_release);
+            lds_limit_raised[half][device].store(true, std::memory_order_release);
         }
-        staircase_pair_kernel<<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
+        if (half) staircase_pair_kernel<_Float16><<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
+        else      staircase_pair_kernel<__bf16><<<(unsigned)grid, kThreads, kPairLdsBytes, stream>>>(P);
     } else if (dtype == MDX_F16) {
         if (narrow) staircase_attn_kernel<_Float16, true><<<(unsigned)grid, kThreads, 0, stream>>>(P);
         else        staircase_attn_kernel<_Float16, false><<<(unsigned)grid, kThreads, 0, stream>>>(P);

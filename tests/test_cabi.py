@@ -115,10 +115,12 @@ def test_context_mirror():
 
 
 def test_generated_kernel_core_is_current():
-    """staircase_pair_core.inc is the committed output of its generator: regenerate and compare."""
+    """staircase_pair_core.inc and its fp16 twin are the committed outputs of their generator: regenerate and compare."""
     import subprocess
     import sys
     from pathlib import Path
     csrc = Path(__file__).resolve().parents[1] / "mineru-diffusion_amd" / "csrc"
     out = subprocess.run([sys.executable, str(csrc / "gen_staircase_pair_core.py")], capture_output=True, text=True, check=True)
     assert out.stdout == (csrc / "staircase_pair_core.inc").read_text()
+    out = subprocess.run([sys.executable, str(csrc / "gen_staircase_pair_core.py"), "f16"], capture_output=True, text=True, check=True)
+    assert out.stdout == (csrc / "staircase_pair_core_f16.inc").read_text()

@@ -411,7 +411,18 @@ def test_fp16_prefill_and_decode(dev, hq, hkv):
     assert o.dtype == torch.float16
     ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
     assert (o.float().cpu() - ref).abs().max().item() < TOL
-    # against the bf16 kernel on the same values rounded to bf16: two roundings apart at most
+    # the pair kernel's fp16 core (even head ratios, sequences beyond a few hundred tokens): other block sizes, a
+    # sequence that ends inside a row group, scores of up to 20 sigma
+    for S, lens2, gain in ((4, [2100, 777], 1.0), (128, [1300, 600, 95], 1.0), (32, [1500], 2.5)):
+        N2 = sum(lens2)
+        q2 = (torch.randn(N2, hq, 128, generator=g) * gain).half()
+        k2 = (torch.randn(N2, hkv, 128, generator=g) * gain).half()
+        v2 = torch.randn(N2, hkv, 128, generator=g).half()
+        cu2 = torch.tensor([0] + list(np.cumsum(lens2)), dtype=torch.int32)
+        o2 = mdx.sparse_attn_varlen(q2.to(dev), k2.to(dev), v2.to(dev), cu2.to(dev), cu2.to(dev), S)
+        ref2 = oracle.staircase_attn_varlen(q2, k2, v2, cu2, S)
+        err = (o2.float().cpu() - ref2).abs().max().item()
+        assert err < TOL, f"fp16 S={S} lens={lens2}: max-abs {err}"
     for ctxs in ([700, 4128, 33], [2300] * 4):
         qd, kc, vc, bt, lens_d = _paged_inputs(g, ctxs, hq=hq, hkv=hkv)
         qd, kc, vc = qd.half(), kc.half(), vc.half()
