@@ -269,6 +269,36 @@ def test_attention_with_peaked_scores(dev, scale_qk, hq, hkv, S):
     assert err < 1.5 * TOL, err
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_prefill_one_dominant_key_anywhere_in_a_tile(dev, dtype):
+    """One key per sequence scores some 300 octaves above every other: wherever in its 64-key tile it lies, the
+    running maximum has to move before the exponentials of that tile (else the probability overflows: the limit is
+    2^16 in fp16 and 2^128 in bf16) and what was accumulated before it has to vanish.  Sequence i of the first 64 has
+    the key at padded position 64 + i (the tile after the one that holds the padding, whose iteration applies the
+    key mask), sequence 64 + i has it i keys before the end (tiles on the staircase's edge)."""
+    import mdx
+    g = torch.Generator().manual_seed(77)
+    L, n = 601, 128
+    pad = (-L) % 32
+    lens = [L] * n
+    q = torch.randn(n * L, 2, 128, generator=g) * 0.25 + 3.0
+    k = torch.randn(n * L, 1, 128, generator=g) * 0.25
+    v = torch.randn(n * L, 1, 128, generator=g)
+    where = [64 + i - pad for i in range(64)] + [L - 1 - i for i in range(64)]
+    for b, j in enumerate(where):
+        k[b * L + j] = 6.0
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32, max_seqlen=1024).float().cpu()
+    ref = oracle.staircase_attn_varlen(q, k, v, cu, 32)
+    assert torch.isfinite(o).all()
+    err = (o - ref).abs().amax(dim=(1, 2)).view(n, L).amax(dim=1)
+    assert err.max().item() < TOL, f"max-abs {err.max().item()} in sequence {int(err.argmax())} (key at {where[int(err.argmax())]})"
+    for b, j in enumerate(where):                      # the rows that see the key return its value row
+        first = min(L, ((j + pad) // 32 + 1) * 32 - pad) - 1
+        assert (o[b * L + first] - v[b * L + j].float()).abs().max().item() < TOL
+
+
 def test_attention_with_uniformly_low_and_constant_scores(dev):
     """All scores equal (K = 0: the output is the mean of the visible V rows) and all scores far
     below zero (q = -k direction): nothing in the kernels may depend on the scores' absolute level."""
