@@ -18,22 +18,23 @@ HEADS = [(16, 8), (8, 8), (4, 1), (6, 3), (3, 1), (2, 1), (12, 4)]
 def test_prefill_random_shapes(dev):
     import mdx
     rng = np.random.default_rng(2024)
-    for case in range(24):
+    for case in range(36):
+        dtype = torch.bfloat16 if case < 24 else torch.float16     # the reference kernel computes in q's dtype
         hq, hkv = HEADS[rng.integers(len(HEADS))]
         S = int(2 ** rng.integers(0, 8))
         B = int(rng.integers(1, 7))
         lens = [int(x) for x in rng.integers(0, 400, B)]
-        if case % 4 == 0:
+        if case % 4 == 0 or case >= 30:
             lens[rng.integers(B)] = int(rng.integers(400, 1500))
         if sum(lens) == 0:
             lens[0] = 5
         g = torch.Generator().manual_seed(1000 + case)
         N = sum(lens)
-        q = torch.randn(N, hq, 128, generator=g).bfloat16()
-        k = torch.randn(N, hkv, 128, generator=g).bfloat16()
-        v = torch.randn(N, hkv, 128, generator=g).bfloat16()
+        q = torch.randn(N, hq, 128, generator=g).to(dtype)
+        k = torch.randn(N, hkv, 128, generator=g).to(dtype)
+        v = torch.randn(N, hkv, 128, generator=g).to(dtype)
         cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
-        print(f"prefill case {case}: heads {hq}/{hkv} S {S} lens {lens}", flush=True)
+        print(f"prefill case {case}: {dtype} heads {hq}/{hkv} S {S} lens {lens}", flush=True)
         o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S)
         torch.cuda.synchronize()
         ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
