@@ -371,13 +371,27 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
 #pragma unroll
                 for (int i = 0; i < EPC; ++i) offer(x[i], c0 + i, g[i]);
             } else if (whole_groups) {
+                U4 r[EPC / 4];
+#pragma unroll
+                for (int q = 0; q < EPC / 4; ++q) r[q] = rn.group((uint32_t)(c0 >> 2) + q);
+                // The generator's bits decide before any logarithm is taken.  An element reaches the lead only with
+                // noise -ln(-ln u) >= need = lead - (largest element) / T, i.e. -ln u <= e^-need; and -ln u >= 1 - u
+                // = (j + 1/2) 2^-23, where j = ~bits >> 9 counts u down from its largest value.  So only draws with
+                // j <= e^-need 2^23 matter: at need = 10, one in 22 000.  need is taken 0.02 + 2^-22 |lead| lower than
+                // computed, which covers the error of the hardware logarithms (2e-6) and every rounding on the way.
+                const float lim = fmaxf(best, seen);
+                const float need = lim - (unit_T ? cmx : cmx / T_) - __builtin_fmaf(fabsf(lim), 2.384185791015625e-07f, 0.02f);
+                const float reach = fminf(fast_exp2(__builtin_fmaf(-kLog2e, need, 23.f)), 8388608.f);    // NaN (lead and element both infinite) -> the other operand
+                uint32_t top = 0;
+#pragma unroll
+                for (int q = 0; q < EPC / 4; ++q) top = max(max(top, max(r[q].x, r[q].y)), max(r[q].z, r[q].w));
+                if (__builtin_amdgcn_ballot_w64((~top >> 9) <= (uint32_t)reach + 1u) == 0) continue;
 #pragma unroll
                 for (int q = 0; q < EPC / 4; ++q) {
-                    const U4 r = rn.group((uint32_t)(c0 >> 2) + q);
-                    offer(x[4 * q + 0], c0 + 4 * q + 0, gumbel_of(r.x));
-                    offer(x[4 * q + 1], c0 + 4 * q + 1, gumbel_of(r.y));
-                    offer(x[4 * q + 2], c0 + 4 * q + 2, gumbel_of(r.z));
-                    offer(x[4 * q + 3], c0 + 4 * q + 3, gumbel_of(r.w));
+                    offer(x[4 * q + 0], c0 + 4 * q + 0, gumbel_of(r[q].x));
+                    offer(x[4 * q + 1], c0 + 4 * q + 1, gumbel_of(r[q].y));
+                    offer(x[4 * q + 2], c0 + 4 * q + 2, gumbel_of(r[q].z));
+                    offer(x[4 * q + 3], c0 + 4 * q + 3, gumbel_of(r[q].w));
                 }
             } else {
 #pragma unroll
