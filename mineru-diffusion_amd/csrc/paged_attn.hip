@@ -37,7 +37,8 @@ namespace {
 using namespace mdx_attn;
 
 constexpr int kMaxSq = 32;
-constexpr int kChunkAlign = 256;   // split boundaries are multiples of this many keys
+constexpr int kChunkAlign = 256;   // the host's split sizes are multiples of this many keys
+constexpr int kCUs = 256;          // MI355X
 
 // Sum over the 64 lanes: DPP shifts inside the rows of 16 lanes, the two row broadcasts, the total from lane 63
 // (six additions, no LDS traffic: the butterfly of cross-lane LDS permutes it replaces sat in every workgroup's start).
@@ -86,6 +87,14 @@ struct PagedParams {
     // through the scalar cache and wait on the vector-memory counter for them, draining the K/V
     // prefetch queue (measured: 78 -> 120 us).  Split sizes are far below 2^24, so the value is exact.
     float* span_out;
+    // > 0: every sequence is cut (fewer (sequence, head group) pairs than the chip holds workgroups) and the host's
+    // split assumes page tables that are 65 % full.  The attention kernel, which sees the lengths, grows the split
+    // by a tile at a time until the launch fits this many resident workgroups -- one round, nobody starts late --
+    // and leaves the split it settled on in span_out.  (Full tables: 16 sequences of 4128 keys 69 -> 60 us, 16 of
+    // 1000 to 3000 keys in a table 12 pages wide 51 -> 42 us; no shape of the sweep slower.  Cutting each sequence
+    // into equal pieces instead of full splits and a short remainder was measured too and loses: the remainders
+    // start last and fill the tail.)
+    int fit_slots;
     // Single-launch mode: one arrival counter per (sequence, head group), zero between launches.  The
     // last split of a pair to arrive merges the pair's partials itself.  float for the same reason.
     float* arrive;
@@ -201,19 +210,31 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         // lengths beyond the page table name keys that do not exist: clipped here and below
         const int ctx_l = lane < P.bs ? min(max(0, P.context_lens[lane]), P.max_pages * P.page_size) : 0;
         ctx_all = ctx_l;
-        if (P.span_out) {
-            // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
-            // nothing to combine) -- unless one of them is much longer than the rest and would keep
-            // its CU busy long after the others are done.  Only the device knows the lengths: the
-            // split grows from the host's size to 1.25 x the mean length, so that only sequences
-            // well above the mean are cut, into pieces of about the mean.
-            const int live = wave_sum(ctx_l > 0 ? 1 : 0);
-            const int mean = wave_sum(ctx_l) / max(live, 1);
-            span = max(span, (mean + mean / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
+        auto splits_of_lane = [&]() { return lane < P.bs ? max(1, (ctx_l + span - 1) / span) : 0; };   // (padding rows get one)
+        int n;
+        if (P.fit_slots > 0) {
+            n = splits_of_lane();
+            // a tile more per step (24 steps double the smallest split); a few workgroups beyond what is resident
+            // may stay: the last to start are remainders, which fill the tail
+            for (int it = 0; it < 24 && wave_sum(n) * (int)gridDim.x > P.fit_slots + P.fit_slots / 32; ++it) {
+                span += 64;
+                n = splits_of_lane();
+            }
             if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
+        } else {
+            if (P.span_out) {
+                // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
+                // nothing to combine) -- unless one of them is much longer than the rest and would keep
+                // its CU busy long after the others are done.  Only the device knows the lengths: the
+                // split grows from the host's size to 1.25 x the mean length, so that only sequences
+                // well above the mean are cut, into pieces of about the mean.
+                const int live = wave_sum(ctx_l > 0 ? 1 : 0);
+                const int mean = wave_sum(ctx_l) / max(live, 1);
+                span = max(span, (mean + mean / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
+                if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
+            }
+            n = splits_of_lane();
         }
-        int n = 0;                                  // splits of sequence `lane` (padding rows get one)
-        if (lane < P.bs) n = max(1, (ctx_l + span - 1) / span);
         // Launch order: the first split of every sequence, then the second of those that have one, ...
         // The last split of a sequence is its short remainder, so the workgroups that start late
         // (when there are more of them than the chip holds at once) are the short ones.
@@ -575,7 +596,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     P.num_q_heads = num_q_heads;
     P.head_dim = head_dim;
     P.c = scale * kLog2e;
-    P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr; P.arrive = nullptr;
+    P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr; P.arrive = nullptr; P.fit_slots = 0;
     if (P.nsplit > 1) {
         const int64_t n_slots = (int64_t)bs * num_q_heads * P.nsplit;
         const int64_t need = n_slots * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;
@@ -584,7 +605,8 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
         MDX_REQUIRE(mdx::aligned16(workspace), MDX_EWORKSPACE, "paged_block_attn: workspace not 16-byte aligned");
         P.part_o = static_cast<float*>(workspace);
         P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
-        if (device_span) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
+        if (!device_span && bs <= 64) P.fit_slots = kCUs * (HPW == 2 ? 2 : 1);       // workgroups resident at once
+        if (device_span || P.fit_slots > 0) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
         // Single launch: the partials are written through with agent-scope stores and read back with
         // agent-scope loads, so counting in costs a workgroup the wait for its own stores and one atomic,
         // not a device-wide release (a write-back walk of its XCD's L2).  Where only outliers are cut

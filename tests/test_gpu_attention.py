@@ -214,6 +214,14 @@ def test_paged_config2_shape(dev):
     _check_paged(dev, ctxs, seed=2, pool=300)
 
 
+@pytest.mark.parametrize("ctxs", [[4128] * 16, [3072, 2900, 1000] * 5, [4352] * 9 + [40, 0, 700]])
+def test_paged_full_tables_grow_the_split_on_the_device(dev, ctxs):
+    """Page tables far fuller than the host's split size assumes: the attention kernel grows the split from the
+    lengths until the launch fits the chip in one round and tells the combine kernel; the result does not depend on
+    where the splits fall (fp32 oracle, max-abs < 2e-2; the single launch and the two launches agree bit for bit)."""
+    _check_paged(dev, ctxs, seed=len(ctxs), pool=sum((c + 255) // 256 for c in ctxs) + 4)
+
+
 def test_decode_matches_prefill_last_block(dev):
     """Cross-check of the two kernels: prefill of (prefix + block) then decode of the same block over
     the stored cache must agree (the decode block sees prefix + itself, as the last prefill block does)."""
