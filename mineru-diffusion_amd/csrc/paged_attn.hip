@@ -53,6 +53,17 @@ __device__ __forceinline__ int wave_sum(int x) {
     return __builtin_amdgcn_readlane(v, 63);
 }
 
+__device__ __forceinline__ int wave_max(int x) {                         // same pattern; x >= 0
+    int v = x;
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false));
+    return __builtin_amdgcn_readlane(v, 63);
+}
+
 // Partials that another workgroup of the same launch reads (single-launch merge) travel with
 // agent-scope accesses: such a store is written through to memory and such a load does not take a line
 // that this XCD's L2 may still hold from an earlier launch.  That makes them visible across the XCDs'
@@ -88,9 +99,9 @@ struct PagedParams {
     // prefetch queue (measured: 78 -> 120 us).  Split sizes are far below 2^24, so the value is exact.
     float* span_out;
     // > 0: every sequence is cut (fewer (sequence, head group) pairs than the chip holds workgroups) and the host's
-    // split assumes page tables that are 65 % full.  The attention kernel, which sees the lengths, grows the split
-    // by a tile at a time until the launch fits this many resident workgroups -- one round, nobody starts late --
-    // and leaves the split it settled on in span_out.  (Full tables: 16 sequences of 4128 keys 69 -> 60 us, 16 of
+    // split assumes page tables that are 65 % full.  The attention kernel, which sees the lengths, starts from the
+    // split that fills the chip when the tables are emptier, grows it by a tile at a time until the launch fits this
+    // many resident workgroups -- one round, nobody starts late -- and leaves the split it settled on in span_out.  (Full tables: 16 sequences of 4128 keys 69 -> 60 us, 16 of
     // 1000 to 3000 keys in a table 12 pages wide 51 -> 42 us; no shape of the sweep slower.  Cutting each sequence
     // into equal pieces instead of full splits and a short remainder was measured too and loses: the remainders
     // start last and fill the tail.)
@@ -213,6 +224,16 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         auto splits_of_lane = [&]() { return lane < P.bs ? max(1, (ctx_l + span - 1) / span) : 0; };   // (padding rows get one)
         int n;
         if (P.fit_slots > 0) {
+            // Tables emptier than assumed: start from the split that would fill the chip -- at least 512 keys, no more
+            // pieces per sequence than the launch has room for, and only if that takes 256 keys or more off the
+            // longest workgroup (what a combine pass and the partials cost).
+            const int total = wave_sum(ctx_l), longest = wave_max(ctx_l), live = wave_sum(ctx_l > 0 ? 1 : 0);
+            // (quotients by reciprocal: an estimate is all that is needed, and every workgroup makes the same one; the
+            // "+ 1" keeps the longest sequence within nsplit pieces whatever the rounding)
+            const float room = fmaxf(1.f, (float)P.fit_slots * __builtin_amdgcn_rcpf((float)gridDim.x) - 0.5f * (float)live);   // pieces; a remainder of half a split per sequence
+            const int fill = max(max(512, ((int)((float)total * __builtin_amdgcn_rcpf(room)) + 63) & ~63),
+                                 ((int)((float)longest * __builtin_amdgcn_rcpf((float)P.nsplit)) + 1 + 63) & ~63);
+            if (min(longest, span) - fill >= 256) span = fill;
             n = splits_of_lane();
             // a tile more per step (24 steps double the smallest split); a few workgroups beyond what is resident
             // may stay: the last to start are remainders, which fill the tail
@@ -504,7 +525,8 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // are about as many (sequence, head group) pairs as CUs (from 192 pairs on) (in the engine's decode pass at batch 32 that beats two
 // splits per sequence by 4 %: no partials to write, nothing to combine).  The host knows the
 // page-table width, not the lengths: tables are taken to be about 65 % full, and the last split of
-// a sequence to be half a split.  In the pair-per-CU case up to four splits per sequence are allowed
+// a sequence to be half a split (the attention kernel, which sees the lengths, corrects the split
+// both ways: PagedParams::fit_slots).  In the pair-per-CU case up to four splits per sequence are allowed
 // and the kernel itself, which sees the lengths, cuts only sequences well above the mean
 // (*device_span; the dense workgroup numbering that this needs exists for up to 64 sequences).
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* device_span) {

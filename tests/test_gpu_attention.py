@@ -222,6 +222,26 @@ def test_paged_full_tables_grow_the_split_on_the_device(dev, ctxs):
     _check_paged(dev, ctxs, seed=len(ctxs), pool=sum((c + 255) // 256 for c in ctxs) + 4)
 
 
+@pytest.mark.parametrize("ctxs,width", [([1000] * 8, 32), ([537, 1490, 800, 1203, 640, 0, 1111, 999] * 2, 32), ([2000] * 4, 64),
+                                        ([600] * 16, 17), ([3000, 5, 2900] * 2, 64)])
+def test_paged_wide_tables_shrink_the_split_on_the_device(dev, ctxs, width):
+    """Page tables much wider than the contexts: the host's split (sized for tables 65 % full) would leave most of
+    the chip idle; the kernel starts from the split that fills it (not below 512 keys, not where too little is
+    gained) -- same results."""
+    import mdx
+    g = torch.Generator().manual_seed(width + len(ctxs))
+    q, kc, vc, bt, lens = _paged_inputs(g, ctxs, pool=sum((c + 255) // 256 for c in ctxs) + 4)
+    wide = torch.full((len(ctxs), width), -1, dtype=torch.int32)
+    wide[:, :bt.shape[1]] = bt
+    scale = 1 / math.sqrt(128)
+    kw = dict(cache_seqlens=lens.to(dev), block_table=wide.to(dev), softmax_scale=scale, causal=False)
+    o = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), **kw)
+    ref = oracle.paged_block_attn(q, kc, vc, bt, lens, scale)
+    assert (o.float().cpu() - ref).abs().max().item() < TOL
+    two = mdx.flash_attn_with_kvcache(q.to(dev), kc.to(dev), vc.to(dev), counters=False, **kw)
+    assert torch.equal(o, two)
+
+
 def test_decode_matches_prefill_last_block(dev):
     """Cross-check of the two kernels: prefill of (prefix + block) then decode of the same block over
     the stored cache must agree (the decode block sees prefix + itself, as the last prefill block does)."""
