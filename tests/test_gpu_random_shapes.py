@@ -62,6 +62,8 @@ def test_paged_random_shapes(dev):
         if max(ctxs) == 0:
             ctxs[0] = 3
         extra = int(rng.integers(0, 3))                         # unused table columns (-1)
+        if case % 4 == 1:
+            extra += int(rng.integers(8, 48))                   # a table far wider than the contexts (the kernel then re-sizes the splits)
         pages = [(c + page - 1) // page for c in ctxs]
         pool = sum(pages) + 3
         g = torch.Generator().manual_seed(2000 + case)
