@@ -224,16 +224,27 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         auto splits_of_lane = [&]() { return lane < P.bs ? max(1, (ctx_l + span - 1) / span) : 0; };   // (padding rows get one)
         int n;
         if (P.fit_slots > 0) {
-            // Tables emptier than assumed: start from the split that would fill the chip -- at least 512 keys, no more
-            // pieces per sequence than the launch has room for, and only if that takes 256 keys or more off the
-            // longest workgroup (what a combine pass and the partials cost).
+            // Tables emptier than assumed: start from the split that would fill the chip, total / (resident workgroups
+            // per head group - a remainder of half a split per sequence) -- at least 512 keys (256 where even pieces
+            // that short leave half of the chip's workgroup slots empty: a launch that small is a chain of
+            // latencies, and the chain is as long as its longest workgroup), no more pieces per sequence than the
+            // launch has room for, and not so many that the combine pass, which walks a sequence's pieces four at a
+            // time, costs more than shorter pieces save (0.6 us per piece against 0.022 us per key of the longest
+            // workgroup: pieces of sqrt(27.6 x longest) keys balance the two; a sequence of tens of thousands of
+            // keys grows its split by the same rule).  A sequence that the host's split leaves whole is only cut
+            // if that takes 256 keys or more off the longest workgroup (what the combine pass and the partials cost).
+            // (Quotients by reciprocal: an estimate is all that is needed, and every workgroup makes the same one;
+            // the "+ 1" keeps the longest sequence within nsplit pieces whatever the rounding.)
             const int total = wave_sum(ctx_l), longest = wave_max(ctx_l), live = wave_sum(ctx_l > 0 ? 1 : 0);
-            // (quotients by reciprocal: an estimate is all that is needed, and every workgroup makes the same one; the
-            // "+ 1" keeps the longest sequence within nsplit pieces whatever the rounding)
-            const float room = fmaxf(1.f, (float)P.fit_slots * __builtin_amdgcn_rcpf((float)gridDim.x) - 0.5f * (float)live);   // pieces; a remainder of half a split per sequence
-            const int fill = max(max(512, ((int)((float)total * __builtin_amdgcn_rcpf(room)) + 63) & ~63),
-                                 ((int)((float)longest * __builtin_amdgcn_rcpf((float)P.nsplit)) + 1 + 63) & ~63);
-            if (min(longest, span) - fill >= 256) span = fill;
+            const float per_group = (float)P.fit_slots * __builtin_amdgcn_rcpf((float)gridDim.x);      // resident workgroups per head group
+            const float room = fmaxf(1.f, per_group - 0.5f * (float)live);
+            const float least = (float)total * (1.f / 256.f) + (float)live <= 0.5f * per_group ? 256.f : 512.f;
+            const float depth = __builtin_amdgcn_sqrtf(27.6f * (float)longest);
+            const float want = fmaxf(fmaxf(least, (float)total * __builtin_amdgcn_rcpf(room)),
+                                     fmaxf((float)longest * __builtin_amdgcn_rcpf((float)P.nsplit) + 1.f, depth));
+            const int fill = ((int)want + 63) & ~63;
+            if (min(longest, span) - fill >= (longest > span ? 64 : 256)) span = fill;
+            span = max(span, ((int)depth + 63) & ~63);
             n = splits_of_lane();
             // a tile more per step (24 steps double the smallest split); a few workgroups beyond what is resident
             // may stay: the last to start are remainders, which fill the tail
