@@ -20,6 +20,7 @@ import json
 import math
 import os
 import sys
+import threading
 import time
 from itertools import count
 from pathlib import Path
@@ -108,6 +109,79 @@ def op_entry(ms_graph, ms_single, bound, work, unit_div, peak, unit, extra=None)
 
 def raw_stream():
     return torch.cuda.current_stream().cuda_stream
+
+
+class PowerSampler:
+    """Reads the socket power (hwmon power1_input, microwatts) and the shader clock (the starred line
+    of pp_dpm_sclk) of card 0 from sysfs every few milliseconds on a host thread while a leg runs.
+    Read-only files that an ordinary user may read; where they are missing the leg reports that."""
+
+    def __init__(self, period_s=0.005):
+        self.period = period_s
+        self.power_file = self.sclk_file = self.cap_w = None
+        for dev_dir in sorted(Path("/sys/class/drm").glob("card*/device")):
+            for hw in sorted(dev_dir.glob("hwmon/hwmon*")):
+                if (hw / "power1_input").exists() or (hw / "power1_average").exists():
+                    self.power_file = hw / ("power1_input" if (hw / "power1_input").exists() else "power1_average")
+                    if (hw / "power1_cap").exists():
+                        try:
+                            self.cap_w = int((hw / "power1_cap").read_text()) / 1e6
+                        except (OSError, ValueError):
+                            pass
+                    if (dev_dir / "pp_dpm_sclk").exists():
+                        self.sclk_file = dev_dir / "pp_dpm_sclk"
+                    break
+            if self.power_file is not None:
+                break
+
+    def available(self):
+        return self.power_file is not None
+
+    def _read(self):
+        w = mhz = None
+        try:
+            w = int(self.power_file.read_text()) / 1e6
+        except (OSError, ValueError):
+            pass
+        if self.sclk_file is not None:
+            try:
+                for line in self.sclk_file.read_text().splitlines():
+                    if line.rstrip().endswith("*"):
+                        mhz = float(line.split(":")[1].strip().split("M")[0])
+            except (OSError, ValueError, IndexError):
+                pass
+        return w, mhz
+
+    def run(self, enqueue, seconds):
+        """Calls enqueue() (which replays a HIP graph of back-to-back launches and synchronizes) in a loop for
+        about `seconds` while the thread samples; returns mean / max power and clock over the samples taken
+        after the first third of the time (ramp), and the average duration of one enqueue() in that part."""
+        samples, stop = [], threading.Event()
+
+        def sample():
+            while not stop.is_set():
+                samples.append((time.perf_counter(),) + self._read())
+                time.sleep(self.period)
+        th = threading.Thread(target=sample, daemon=True)
+        th.start()
+        t0 = time.perf_counter()
+        marks = []
+        while time.perf_counter() - t0 < seconds:
+            enqueue()
+            marks.append(time.perf_counter())
+        stop.set()
+        th.join()
+        cut = t0 + seconds / 3
+        late = [s for s in samples if s[0] >= cut]
+        ws = [s[1] for s in late if s[1] is not None]
+        cs = [s[2] for s in late if s[2] is not None]
+        late_marks = [m for m in marks if m >= cut]
+        per_call = (late_marks[-1] - late_marks[0]) / (len(late_marks) - 1) if len(late_marks) > 1 else float("nan")
+        return dict(samples=len(late), power_w_mean=round(float(np.mean(ws)), 1) if ws else None,
+                    power_w_max=round(float(np.max(ws)), 1) if ws else None,
+                    sclk_mhz_mean=round(float(np.mean(cs)), 1) if cs else None,
+                    sclk_mhz_min=round(float(np.min(cs)), 1) if cs else None,
+                    sclk_mhz_max=round(float(np.max(cs)), 1) if cs else None), per_call
 
 
 # ----------------------------------------------------------------------------- config 3
@@ -383,7 +457,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-full-logits-leg", action="store_true",
                     help="decode leg: skip the second generation that projects all 32 positions of every block")
-    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,decode (default all; gumbel and filter run inside unmask)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,decode (default all; gumbel and filter run inside unmask), plus power (only when named: socket power and clock under the attention kernel and the library GEMM)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -466,6 +540,49 @@ def main():
             calibration["staircase_attn_zero_inputs"] = dict(tflops=round(work3["flops"] / z_ms / 1e9, 1), ms=round(z_ms, 4))
             del zf
             del z
+    power = None
+    if "power" in only:
+        # Socket power and shader clock while the attention kernel (and, beside it, the library GEMM) runs back to
+        # back for a few seconds each, on N(0,1) data and on zeros: the evidence for "the clock is power-limited and
+        # operand bit toggling sets the power".  Off by default (it adds 15 s); profiles/ keeps a summary of one run.
+        ps = PowerSampler()
+        if not ps.available():
+            power = {"error": "no readable hwmon power file under /sys/class/drm/card*/device"}
+        else:
+            power = {"power_cap_w": ps.cap_w, "source": f"{ps.power_file} and {ps.sclk_file}, sampled every 5 ms on a host thread; "
+                     "figures are over the last two thirds of a 3 s loop of HIP-graph replays (20 launches each)"}
+            time.sleep(1.0)
+            idle_w, idle_mhz = ps._read()
+            power["idle"] = dict(power_w=idle_w, sclk_mhz=idle_mhz)
+            zf = torch.zeros(g3["q"].shape[0], (HQ + 2 * HKV) * D, dtype=torch.bfloat16, device=dev)
+            z = (torch.zeros_like(g3["q"]), torch.zeros_like(g3["k"]), zf[:, (HQ + HKV) * D:].view(-1, HKV, D))
+            a_r = torch.randn(8192, 8192, device=dev).bfloat16()
+            a_z = torch.zeros(8192, 8192, device=dev, dtype=torch.bfloat16)
+            gemm_flops = 2 * 8192 ** 3
+            for name, fn, flops in (("staircase_attn_config3_random", lambda: attn_only(0), work3["flops"]),
+                                    ("staircase_attn_config3_zeros", lambda: attn_only(0, z), work3["flops"]),
+                                    ("library_gemm_bf16_8192_random", lambda: torch.matmul(a_r, a_r), gemm_flops),
+                                    ("library_gemm_bf16_8192_zeros", lambda: torch.matmul(a_z, a_z), gemm_flops)):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    for _ in range(20):
+                        fn()
+
+                def replay():
+                    gr.replay()
+                    torch.cuda.synchronize()
+                stats, per_call = ps.run(replay, 3.0)
+                stats["ms_per_launch"] = round(per_call * 1e3 / 20, 4)
+                stats["tflops"] = round(flops / (per_call / 20) / 1e12, 1)
+                power[name] = stats
+                log(f"[bench] power leg {name}: {stats}")
+                del gr
+                time.sleep(0.5)
+            del zf, z, a_r, a_z
+            torch.cuda.empty_cache()
     if want("store"):
         # three rotating (source, cache) sets, about 900 MB touched per round trip, so the 256 MB
         # last-level cache cannot serve the next launch; the C ABI is called directly
@@ -641,6 +758,7 @@ def main():
         "ops": result_ops,
         "calibration": calibration,
         "decode": decode,
+        "power": power,
         "host": {"cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads()},
     }
     print(json.dumps(line), flush=True)

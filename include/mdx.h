@@ -9,8 +9,17 @@
  * until the stream has passed the call); outputs and workspaces are allocated
  * by the caller.  No entry point allocates, frees or synchronises; every
  * kernel is enqueued on `stream` (a hipStream_t, 0 = the null stream), so all
- * of them may be recorded into a HIP graph.  The library keeps no global state
- * apart from a thread-local error string.
+ * of them may be recorded into a HIP graph.
+ *
+ * Global state of the library, all of it: (1) a thread-local error string
+ * (mdx_last_error); (2) per device, set once on the first call that needs it
+ * and never changed afterwards: the raised dynamic-LDS limit of the staircase
+ * pair kernel (a function attribute) and the number of compute units that the
+ * paged attention sizes its splits by; (3) the file-scope __device__ array of
+ * 40 MiB behind mdx_paged_block_attn_static, one copy per GPU, with the
+ * per-device address of it cached after the first call on that device; calls
+ * of that one entry point that overlap on one GPU race on the array.  No other
+ * entry point shares memory between calls: they are re-entrant.
  *
  * Return value: 0 on success, a negative MDX_E* code otherwise (nothing has
  * been enqueued then); mdx_last_error() gives the reason as text.
@@ -121,7 +130,8 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
  * contents need no initialisation.
  * Supported: d a multiple of 16 up to 128 (narrower heads are padded with zeros on the way into LDS; the
- * partials keep their 128-wide layout), Sq <= 32 (any Hq that is a multiple of Hkv), page_size % 32 == 0,
+ * partials keep their 128-wide layout), Sq <= 128 (blocks longer than 32 positions run as tiles of 32 queries
+ * that stream the same keys; any Hq that is a multiple of Hkv), page_size % 32 == 0,
  * MDX_BF16 or MDX_F16.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
@@ -146,7 +156,8 @@ int mdx_paged_block_attn(const void* q, void* o, const void* k_cache, const void
  * fewer pairs, where every sequence is split, the call makes the same two launches as
  * mdx_paged_block_attn (counting in costs each split workgroup a device-wide release).
  *
- * counters: mdx_paged_block_attn_counter_bytes(bs, Hq, Hkv) bytes of device memory, 4-byte
+ * counters: mdx_paged_block_attn_counter_bytes(bs, Hq, Hkv) bytes of device memory (one fp32 per
+ * sequence, head group and tile of 32 queries, sized for Sq = 128), 4-byte
  * aligned, that MUST BE ZERO before the first call and are left zero by every call that
  * completes; calls that may run at the same time (different streams) need counters of their
  * own.  workspace as above.  Same results bit for bit as mdx_paged_block_attn.

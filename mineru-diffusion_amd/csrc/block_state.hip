@@ -76,7 +76,7 @@ __global__ __launch_bounds__(1024) void masked_rows_kernel(
     // the rest of the fixed-size list repeats its first entry (row 0 when nothing is masked): rows
     // computed twice give the same values, so scattering their results back is harmless
     __syncthreads();
-    const int64_t fill = found > 0 ? rows_out[0] : 0;
+    const int64_t fill = (found > 0 && rows_cap > 0) ? rows_out[0] : 0;     // rows_cap == 0: rows_out may be null, only the count is wanted
     for (int i = (found < rows_cap ? found : rows_cap) + tid; i < rows_cap; i += 1024) rows_out[i] = fill;
     if (tid == 0) *n_rows_out = found;
 }

@@ -1,6 +1,11 @@
-// Paged single-block ("decode") attention: the Sq <= 32 queries of the current
+// Paged single-block ("decode") attention: the Sq <= 128 queries of the current
 // denoising block of every sequence attend, non-causally, to the first
-// context_lens[b] keys of that sequence's paged KV cache.
+// context_lens[b] keys of that sequence's paged KV cache.  A workgroup serves one
+// tile of 32 queries; blocks of 64 or 128 positions (the reference's block length
+// is a configuration field, nanovllm/config.py:48) run as 2 or 4 query tiles on
+// the grid's z axis, each with its own partials and arrival counter, and stream
+// the same keys (which the tiles of a pair, launched next to each other, mostly
+// find in the L2 that the first of them filled).
 //
 // Replaces flash_attn_with_kvcache(..., causal=False) at
 // engines/nano_dvlm/nanovllm/layers/sdar_attention.py:48-56.
@@ -31,14 +36,15 @@
 //    (m, l, O) that a second, small kernel combines.
 #include "mdx_common.h"
 #include "attn_tile.h"
+#include <atomic>
 
 namespace {
 
 using namespace mdx_attn;
 
-constexpr int kMaxSq = 32;
+constexpr int kQTile = 32;          // queries per workgroup (one per lane pair of a wavefront)
+constexpr int kMaxSq = 128;         // queries per sequence: up to four query tiles
 constexpr int kChunkAlign = 256;   // the host's split sizes are multiples of this many keys
-constexpr int kCUs = 256;          // MI355X
 
 // Sum over the 64 lanes: DPP shifts inside the rows of 16 lanes, the two row broadcasts, the total from lane 63
 // (six additions, no LDS traffic: the butterfly of cross-lane LDS permutes it replaces sat in every workgroup's start).
@@ -88,10 +94,11 @@ struct PagedParams {
     int bs, sq, heads_per_kv, page_size, page_shift, max_pages;   // page_shift: log2(page_size) or -1
     int64_t num_pages;
     int chunk, nsplit;                              // keys per split, max splits per sequence
+    int nqt;                                        // query tiles of 32 per sequence (grid z)
     int num_q_heads;
     int head_dim;                                   // <= 128, a multiple of 16: columns beyond it are zeros in LDS and never stored
     float c;                                        // scale * log2(e)
-    float* part_o; float* part_ml;                  // [bs, Hq, nsplit, 32, 128] and [bs, Hq, nsplit, 2, 32]
+    float* part_o; float* part_ml;                  // [bs, Hq, nqt, nsplit, 32, 128] and [bs, Hq, nqt, nsplit, 2, 32]
     // non-null: the attention kernel picks the split size (>= chunk) from the lengths and leaves it
     // here for the combine kernel.  A float on purpose: an int store in the attention kernel could
     // alias the int page table and lengths for the compiler, which would then stop fetching those
@@ -117,10 +124,10 @@ struct PagedParams {
 // beyond nv hold leftovers and are masked out), so a caller whose split count is still in flight from
 // memory overlaps that latency with the partials'.
 template <typename E, bool AGENT, typename Count>
-__device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int s, int c, Count count)
+__device__ __forceinline__ void combine_query(const PagedParams& P, int b, int hq, int qt, int s, int c, Count count)
 {
     if (c * 16 >= P.head_dim) return;
-    const int64_t slot0 = ((int64_t)b * P.num_q_heads + hq) * P.nsplit;
+    const int64_t slot0 = (((int64_t)b * P.num_q_heads + hq) * P.nqt + qt) * P.nsplit;
     int nv = P.nsplit;                         // until count() is in: every slot that exists
     float M = kMinusBig, Lsum = 0.f;
     float acc[16];
@@ -132,16 +139,16 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int64_t slot = slot0 + min(i0 + i, P.nsplit - 1);
-            const float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + s;
-            const float* src = P.part_o + (slot * kMaxSq + s) * kHeadDim + c * 16;
+            const float* ml = P.part_ml + (slot * 2 + 0) * kQTile + s;
+            const float* src = P.part_o + (slot * kQTile + s) * kHeadDim + c * 16;
             if (AGENT) {
                 m[i] = __hip_atomic_load(ml, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                l[i] = __hip_atomic_load(ml + kMaxSq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                l[i] = __hip_atomic_load(ml + kQTile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) po[i][k] = load_agent(src + 4 * k);
             } else {
                 m[i] = ml[0];
-                l[i] = ml[kMaxSq];
+                l[i] = ml[kQTile];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) po[i][k] = *reinterpret_cast<const f32x4*>(src + 4 * k);
             }
@@ -182,7 +189,7 @@ __device__ __forceinline__ void combine_query(const PagedParams& P, int b, int h
     }
     const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;   // no valid key at all (every page id invalid): zeros, like a context of 0
     typedef typename Elem16<E>::vec8 vec8;
-    __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
+    __bf16* dst = P.o + (int64_t)b * P.o_sb + (int64_t)(qt * kQTile + s) * P.o_ss + (int64_t)hq * P.o_sh + c * 16;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         vec8 out;
@@ -211,6 +218,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
     const int hg = blockIdx.x;
+    const int qt = blockIdx.z;                      // this workgroup's tile of 32 queries
     const int kw = wave % KW;                       // this wavefront's key slice
     const int head = hg * HPW + wave / KW;          // and query head
 
@@ -236,7 +244,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             // (Quotients by reciprocal: an estimate is all that is needed, and every workgroup makes the same one;
             // the "+ 1" keeps the longest sequence within nsplit pieces whatever the rounding.)
             const int total = wave_sum(ctx_l), longest = wave_max(ctx_l), live = wave_sum(ctx_l > 0 ? 1 : 0);
-            const float per_group = (float)P.fit_slots * __builtin_amdgcn_rcpf((float)gridDim.x);      // resident workgroups per head group
+            const float per_group = (float)P.fit_slots * __builtin_amdgcn_rcpf((float)(gridDim.x * gridDim.z));      // resident workgroups per head group and query tile
             const float room = fmaxf(1.f, per_group - 0.5f * (float)live);
             const float least = (float)total * (1.f / 256.f) + (float)live <= 0.5f * per_group ? 256.f : 512.f;
             const float depth = __builtin_amdgcn_sqrtf(27.6f * (float)longest);
@@ -248,11 +256,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             n = splits_of_lane();
             // a tile more per step (24 steps double the smallest split); a few workgroups beyond what is resident
             // may stay: the last to start are remainders, which fill the tail
-            for (int it = 0; it < 24 && wave_sum(n) * (int)gridDim.x > P.fit_slots + P.fit_slots / 32; ++it) {
+            for (int it = 0; it < 24 && wave_sum(n) * (int)(gridDim.x * gridDim.z) > P.fit_slots + P.fit_slots / 32; ++it) {
                 span += 64;
                 n = splits_of_lane();
             }
-            if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
+            if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) *P.span_out = (float)span;
         } else {
             if (P.span_out) {
                 // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
@@ -263,7 +271,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
                 const int live = wave_sum(ctx_l > 0 ? 1 : 0);
                 const int mean = wave_sum(ctx_l) / max(live, 1);
                 span = max(span, (mean + mean / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
-                if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
+                if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) *P.span_out = (float)span;
             }
             n = splits_of_lane();
         }
@@ -294,7 +302,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     const int n_valid_splits = (ctx + span - 1) / span;
     if (ctx <= 0) {
         // graph-padding row: defined output (zeros), written by its split 0
-        if (split == 0) {
+        if (split == 0 && qt == 0) {
             for (int e = tid; e < P.sq * HPW * (kHeadDim / 8); e += kThreads) {
                 const int d8 = e % (kHeadDim / 8), h = (e / (kHeadDim / 8)) % HPW, s = e / (kHeadDim / 8) / HPW;
                 if (d8 * 8 < P.head_dim) *reinterpret_cast<u32x4*>(P.o + (int64_t)b * P.o_sb + (int64_t)s * P.o_ss + (int64_t)(hg * HPW + h) * P.o_sh + d8 * 8) = u32x4{0, 0, 0, 0};
@@ -307,9 +315,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     const int key_end = min(ctx, key_begin + span);
     const int kvh = (hg * HPW) / P.heads_per_kv;
 
-    const bool row_ok = r < P.sq;
+    const int qrow = qt * kQTile + r;               // this lane's query of the sequence's block
+    const bool row_ok = qrow < P.sq;
     typename Elem16<E>::vec8 q[1][8];
-    load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)r * P.q_ss + (int64_t)head * P.q_sh : nullptr, H, P.head_dim);
+    load_q(q[0], row_ok ? P.q + (int64_t)b * P.q_sb + (int64_t)qrow * P.q_ss + (int64_t)head * P.q_sh : nullptr, H, P.head_dim);
 
     WaveState<1> st;
     st.init();
@@ -452,7 +461,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     if (n_valid_splits == 1) {
         if (!row_ok) return;
         const float inv = st.l[0] > 0.f ? 1.0f / st.l[0] : 0.f;   // no valid key at all: zeros
-        __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)r * P.o_ss + (int64_t)head * P.o_sh;
+        __bf16* orow = P.o + (int64_t)b * P.o_sb + (int64_t)qrow * P.o_ss + (int64_t)head * P.o_sh;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
             if (dt % KW != kw) continue;
@@ -467,8 +476,8 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
         return;
     }
     if (row_ok) {
-        const int64_t slot = ((int64_t)b * P.num_q_heads + head) * P.nsplit + split;
-        float* po = P.part_o + (slot * kMaxSq + r) * kHeadDim;
+        const int64_t slot = (((int64_t)b * P.num_q_heads + head) * P.nqt + qt) * P.nsplit + split;
+        float* po = P.part_o + (slot * kQTile + r) * kHeadDim;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) {
             if (dt % KW != kw) continue;
@@ -480,13 +489,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             }
         }
         if (kw == 0 && H == 0) {
-            float* ml = P.part_ml + (slot * 2 + 0) * kMaxSq + r;
+            float* ml = P.part_ml + (slot * 2 + 0) * kQTile + r;
             if (P.arrive) {
                 __hip_atomic_store(ml, st.m[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(ml + kMaxSq, st.l[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(ml + kQTile, st.l[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else {
                 ml[0] = st.m[0];
-                ml[kMaxSq] = st.l[0];
+                ml[kQTile] = st.l[0];
             }
         }
     }
@@ -500,13 +509,13 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     __shared__ int i_am_last;
     wait_vector_memory();
     __syncthreads();
-    float* counter = P.arrive + (int64_t)b * gridDim.x + hg;
+    float* counter = P.arrive + ((int64_t)b * gridDim.x + hg) * P.nqt + qt;
     if (tid == 0) i_am_last = atomicAdd(counter, 1.0f) == (float)(n_valid_splits - 1) ? 1 : 0;
     __syncthreads();
     if (!i_am_last) return;
     for (int e = tid; e < HPW * 256; e += kThreads) {
         const int s = (e & 255) >> 3;
-        if (s < P.sq) combine_query<E, true>(P, b, hg * HPW + (e >> 8), s, e & 7, [&]() { return n_valid_splits; });
+        if (qt * kQTile + s < P.sq) combine_query<E, true>(P, b, hg * HPW + (e >> 8), qt, s, e & 7, [&]() { return n_valid_splits; });
     }
     if (tid == 0) __hip_atomic_store(counter, 0.f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
 }
@@ -519,10 +528,10 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
 template <typename E>
 __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 {
-    const int hq = blockIdx.x % P.num_q_heads, b = blockIdx.x / P.num_q_heads;
+    const int qt = blockIdx.x % P.nqt, hq = (blockIdx.x / P.nqt) % P.num_q_heads, b = blockIdx.x / P.nqt / P.num_q_heads;
     const int s = threadIdx.x >> 3, c = threadIdx.x & 7;
-    if (s >= P.sq) return;
-    combine_query<E, false>(P, b, hq, s, c, [&]() {
+    if (qt * kQTile + s >= P.sq) return;
+    combine_query<E, false>(P, b, hq, qt, s, c, [&]() {
         const int ctx = min(P.context_lens[b], P.max_pages * P.page_size);
         const int span = P.span_out ? (int)*P.span_out : P.chunk;     // the attention kernel's choice
         return (ctx + span - 1) / span;
@@ -540,19 +549,38 @@ __global__ __launch_bounds__(256) void paged_combine_kernel(const PagedParams P)
 // both ways: PagedParams::fit_slots).  In the pair-per-CU case up to four splits per sequence are allowed
 // and the kernel itself, which sees the lengths, cuts only sequences well above the mean
 // (*device_span; the dense workgroup numbering that this needs exists for up to 64 sequences).
+//
+// The counts behind those rules (1.95 workgroups per CU, pairs per CU) are taken from the current device's
+// number of compute units, read once per device; 256 on the MI355X that the rules were measured on, and
+// where no device can be asked (a shape query in a process without a GPU).
+int cu_count() {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cached[kMaxDevices];
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 256;
+    int n = cached[device].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+        cached[device].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+// head_groups counts the workgroups that one (sequence, split) pair launches: head groups x query tiles.
 int pick_chunk(int bs, int head_groups, int max_pages, int page_size, bool* device_span) {
     *device_span = false;
+    const int cus = cu_count();
     const int64_t max_keys = (int64_t)max_pages * page_size;
     const int64_t whole = (max_keys + kChunkAlign - 1) / kChunkAlign * kChunkAlign;   // one split per sequence
-    const double per_pair = 500.0 / ((double)bs * head_groups) - 0.5;                 // workgroups per pair
-    if ((int64_t)bs * head_groups >= 192 || per_pair <= 1.0) {
+    const double per_pair = 1.953 * cus / ((double)bs * head_groups) - 0.5;           // workgroups per pair
+    if ((int64_t)bs * head_groups >= (cus * 3) / 4 || per_pair <= 1.0) {
         if (bs > 64 || whole < 4 * kChunkAlign) return (int)whole;
         *device_span = true;
         return (int)((whole / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
     }
     int64_t chunk = (int64_t)(0.65 * (double)max_keys / per_pair / kChunkAlign + 0.5) * kChunkAlign;
     if (chunk < 2 * kChunkAlign) chunk = 2 * kChunkAlign;
-    if (2 * chunk >= max_keys && (int64_t)bs * head_groups >= 200) chunk = whole;   // two short splits only to fill CUs
+    if (2 * chunk >= max_keys && (int64_t)bs * head_groups >= (cus * 25) / 32) chunk = whole;   // two short splits only to fill CUs
     return (int)chunk;
 }
 
@@ -570,11 +598,12 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
     if (bs <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pages <= 0 || page_size <= 0) return 0;
     const int G = num_q_heads / num_kv_heads;
     const int HPW = (G % 2 == 0) ? 2 : 1;
+    const int nqt = sq <= kQTile ? 1 : (sq + kQTile - 1) / kQTile;
     bool device_span;
-    const int chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size, &device_span);
+    const int chunk = pick_chunk(bs, num_q_heads / HPW * nqt, max_pages, page_size, &device_span);
     const int nsplit = nsplit_of(max_pages, page_size, chunk);
     if (nsplit <= 1) return 0;
-    return (int64_t)bs * num_q_heads * nsplit * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;   // + the split size
+    return (int64_t)bs * num_q_heads * nqt * nsplit * kQTile * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;   // + the split size
 }
 
 namespace mdx {
@@ -624,22 +653,25 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     P.page_shift = -1;
     for (int i = 0; i < 31; ++i) if (page_size == (1 << i)) P.page_shift = i; P.num_pages = num_pages;
     bool device_span;
-    P.chunk = pick_chunk(bs, num_q_heads / HPW, max_pages, page_size, &device_span);
+    P.nqt = (sq + kQTile - 1) / kQTile;
+    const int64_t wg_per_pair = (int64_t)(num_q_heads / HPW) * P.nqt;               // workgroups of one (sequence, split)
+    const int cus = cu_count();
+    P.chunk = pick_chunk(bs, (int)wg_per_pair, max_pages, page_size, &device_span);
     P.nsplit = nsplit_of(max_pages, page_size, P.chunk);
     P.num_q_heads = num_q_heads;
     P.head_dim = head_dim;
     P.c = scale * kLog2e;
     P.part_o = nullptr; P.part_ml = nullptr; P.span_out = nullptr; P.arrive = nullptr; P.fit_slots = 0;
     if (P.nsplit > 1) {
-        const int64_t n_slots = (int64_t)bs * num_q_heads * P.nsplit;
-        const int64_t need = n_slots * kMaxSq * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;
+        const int64_t n_slots = (int64_t)bs * num_q_heads * P.nqt * P.nsplit;
+        const int64_t need = n_slots * kQTile * (kHeadDim + 2) * (int64_t)sizeof(float) + 16;
         MDX_REQUIRE(workspace && workspace_bytes >= need, MDX_EWORKSPACE,
                     "paged_block_attn: workspace of %lld bytes needed, %lld given", (long long)need, (long long)workspace_bytes);
         MDX_REQUIRE(mdx::aligned16(workspace), MDX_EWORKSPACE, "paged_block_attn: workspace not 16-byte aligned");
         P.part_o = static_cast<float*>(workspace);
-        P.part_ml = P.part_o + n_slots * kMaxSq * kHeadDim;
-        if (!device_span && bs <= 64) P.fit_slots = kCUs * (HPW == 2 ? 2 : 1);       // workgroups resident at once
-        if (device_span || P.fit_slots > 0) P.span_out = P.part_ml + n_slots * kMaxSq * 2;
+        P.part_ml = P.part_o + n_slots * kQTile * kHeadDim;
+        if (!device_span && bs <= 64) P.fit_slots = cus * (HPW == 2 ? 2 : 1);        // workgroups resident at once
+        if (device_span || P.fit_slots > 0) P.span_out = P.part_ml + n_slots * kQTile * 2;
         // Single launch: the partials are written through with agent-scope stores and read back with
         // agent-scope loads, so counting in costs a workgroup the wait for its own stores and one atomic,
         // not a device-wide release (a write-back walk of its XCD's L2).  Where only outliers are cut
@@ -649,7 +681,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
         // 61 us against 49 with the combine launch; with full release fences it was 145), so those
         // launches keep the combine kernel.
         if (single_launch && device_span) {
-            const int64_t need_c = (int64_t)bs * (num_q_heads / HPW) * (int64_t)sizeof(float);
+            const int64_t need_c = (int64_t)bs * wg_per_pair * (int64_t)sizeof(float);
             MDX_REQUIRE(counters && counter_bytes >= need_c, MDX_EWORKSPACE,
                         "paged_block_attn: %lld bytes of arrival counters needed, %lld given", (long long)need_c, (long long)counter_bytes);
             MDX_REQUIRE(((uintptr_t)counters & 3) == 0, MDX_EWORKSPACE, "paged_block_attn: counters not 4-byte aligned");
@@ -661,12 +693,12 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     // With device-chosen splits of at least 1.25 x the mean length, sum_b ceil(len_b / split) <= 1.8 bs:
     // the dense numbering never needs more than 2 bs (sequence, split) pairs, whatever nsplit allows.
     const int pairs_y = device_span ? (bs * P.nsplit < 2 * bs ? bs * P.nsplit : 2 * bs) : bs * P.nsplit;
-    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)pairs_y);
+    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)pairs_y, (unsigned)P.nqt);
     // Up to one (sequence, head group) pair per CU: workgroups of 8 wavefronts on 128-key tiles, so that a
     // CU that holds a single workgroup still has two wavefronts per SIMD (batch 32 x 8 KV heads: 79 -> 69 us
     // on equal lengths); with more pairs than CUs the second round costs more than that gains.
-    const bool eight = device_span && (int64_t)bs * (num_q_heads / HPW) <= 256;
-    const unsigned n_combine = (unsigned)(bs * num_q_heads);
+    const bool eight = device_span && (int64_t)bs * wg_per_pair <= cus;
+    const unsigned n_combine = (unsigned)(bs * num_q_heads * P.nqt);
     const bool two_launches = P.nsplit > 1 && !P.arrive;
     if (dtype == MDX_F16) {
         if (HPW == 2 && eight) paged_block_attn_kernel<_Float16, 2, 2, 8><<<grid, 512, 0, stream>>>(P);
@@ -706,7 +738,8 @@ extern "C" int64_t mdx_paged_block_attn_counter_bytes(int32_t bs, int32_t num_q_
 {
     if (bs <= 0 || num_q_heads <= 0 || num_kv_heads <= 0) return 0;
     const int G = num_q_heads / num_kv_heads;
-    return (int64_t)bs * (num_q_heads / ((G % 2 == 0) ? 2 : 1)) * (int64_t)sizeof(float);
+    // one counter per (sequence, head group, query tile), sized for the largest block (four tiles of 32 queries)
+    return (int64_t)bs * (num_q_heads / ((G % 2 == 0) ? 2 : 1)) * (kMaxSq / kQTile) * (int64_t)sizeof(float);
 }
 
 extern "C" int mdx_paged_block_attn_single_launch(const void* q, void* o, const void* k_cache, const void* v_cache,

@@ -67,7 +67,8 @@ __device__ __forceinline__ void seq_bounds(const StaircaseParams& P, int b, int&
 // fastest, then the sequences that own a row group at this level, and workgroups that find no
 // work may only sit at the very end of the grid.  With up to 64 sequences each wavefront derives
 // this dense numbering itself (lane b holds sequence b's row-group count, lane r evaluates
-// F(r) = #pairs at level >= r); beyond that the grid is the full (level x sequence) rectangle and
+// F(r) = #pairs at level >= r); with more sequences, 64 of them per step, as long as no sequence has more
+// than 64 row groups (8 K tokens); beyond both the grid is the full (level x sequence) rectangle and
 // absent pairs return at once.  Returns false when there is no such pair.
 // Inclusive prefix sum over the 64 lanes of a wavefront (DPP shifts inside rows of 16 lanes, then the
 // two row broadcasts): 6 additions, no LDS traffic.
@@ -84,46 +85,71 @@ __device__ __forceinline__ int wave_prefix_sum(int x)
 }
 
 // `hist`: 65 ints of LDS that belong to the calling wavefront alone (unused when there are more than 64 row groups).
+constexpr int kDenseMaxBatch = 1024;   // sequences per launch that the histogram numbering walks (64 per step)
 __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j, int lane, int* hist, int& b, int& rg)
 {
-    if (P.batch <= 64) {
-        int g = 0;                                             // row groups of sequence `lane`
-        if (lane < P.batch) {
+    // row groups of sequence s (0 for an empty or absent one); never more than the launch has levels for
+    auto groups_of = [&](int s) {
+        int g = 0;
+        if (s < P.batch) {
             int first, len;
-            seq_bounds(P, lane, first, len);
-            if (len > 0) g = ((((len + (1 << P.log2_s) - 1) >> P.log2_s) << P.log2_s) + kRowsPerWg - 1) / kRowsPerWg;
+            seq_bounds(P, s, first, len);
+            if (len > 0) g = min(P.n_row_groups, ((((len + (1 << P.log2_s) - 1) >> P.log2_s) << P.log2_s) + kRowsPerWg - 1) / kRowsPerWg);
         }
+        return g;
+    };
+    if (P.n_row_groups <= 64 && P.batch <= kDenseMaxBatch) {
+        // F(r) = sum over sequences of max(0, g - r) for all 64 levels r at once, without a loop over the
+        // sequences (which took 0.9 us of every workgroup's start at 32 sequences, 1.8 at 64): count the
+        // sequences per value of g (LDS atomics of this wavefront only, which complete in order; 64 sequences
+        // per step, so a prefill of the scheduler's 512 sequences, config.py:38, takes 8 steps), then
+        // C(r) = #{g > r} and F(r) = C(r) + C(r + 1) + ... are two prefix sums with the levels laid out
+        // backwards over the lanes (lane l = level 63 - l).
+        hist[lane] = 0;
+        if (lane == 0) hist[64] = 0;
+        const int g0 = groups_of(lane);
+        if (lane < P.batch) atomicAdd(&hist[g0], 1);
+        for (int s0 = 64; s0 < P.batch; s0 += 64)
+            if (s0 + lane < P.batch) atomicAdd(&hist[groups_of(s0 + lane)], 1);
+        __builtin_amdgcn_wave_barrier();
+        const int c = wave_prefix_sum(hist[64 - lane]);        // C(63 - lane)
+        const int f = wave_prefix_sum(c);                      // F(63 - lane)
+        const unsigned long long above = __ballot(f > j);      // the levels 0 .. n - 1: the high lanes
+        const int n = __popcll(above);
+        if (n == 0) return false;                              // past the last pair
+        const int level = n - 1;
+        // index among the sequences that have this row group: the levels above account for F(level) - C(level) pairs
+        int nth = j - __builtin_amdgcn_readlane(f, 64 - n) + __builtin_amdgcn_readlane(c, 64 - n);
+        b = -1;
+        for (int s0 = 0; s0 < P.batch; s0 += 64) {
+            const int g = s0 == 0 ? g0 : groups_of(s0 + lane);
+            const unsigned long long owners = __ballot(g > level);
+            const int here = __popcll(owners);
+            if (nth < here) {
+                const int before = __popcll(owners & ((1ull << lane) - 1ull));
+                const unsigned long long hit = __ballot(((owners >> lane) & 1ull) != 0 && before == nth);
+                b = s0 + __ffsll((long long)hit) - 1;
+                break;
+            }
+            nth -= here;
+        }
+        rg = level;
+        return b >= 0;
+    }
+    if (P.batch <= 64) {
+        // sequences longer than 64 row groups (8 K tokens): the levels are walked 64 at a time
+        const int g = groups_of(lane);
         int level = -1, f_level = 0;
-        if (P.n_row_groups <= 64) {
-            // F(r) = sum over sequences of max(0, g - r) for all 64 levels r at once, without a loop over the
-            // sequences (which took 0.9 us of every workgroup's start at 32 sequences, 1.8 at 64): count the
-            // sequences per value of g (LDS atomics of this wavefront only, which complete in order), then
-            // C(r) = #{g > r} and F(r) = C(r) + C(r + 1) + ... are two prefix sums with the levels laid out
-            // backwards over the lanes (lane l = level 63 - l).
-            hist[lane] = 0;
-            if (lane == 0) hist[64] = 0;
-            if (lane < P.batch) atomicAdd(&hist[g], 1);        // g <= n_row_groups <= 64
-            __builtin_amdgcn_wave_barrier();
-            const int c = wave_prefix_sum(hist[64 - lane]);    // C(63 - lane)
-            const int f = wave_prefix_sum(c);                  // F(63 - lane)
-            const unsigned long long above = __ballot(f > j);  // the levels 0 .. n - 1: the high lanes
+        for (int base = 0; base < P.n_row_groups; base += 64) {
+            const int r_lane = base + lane;
+            int f = 0;
+            for (int s = 0; s < P.batch; ++s) f += max(0, __builtin_amdgcn_readlane(g, s) - r_lane);
+            const unsigned long long above = __ballot(f > j);  // F decreases with the level: low lanes
+            if (above == 0) break;
             const int n = __popcll(above);
-            if (n > 0) {
-                level = n - 1;
-                f_level = __builtin_amdgcn_readlane(f, 64 - n);
-            }
-        } else {
-            for (int base = 0; base < P.n_row_groups; base += 64) {
-                const int r_lane = base + lane;
-                int f = 0;
-                for (int s = 0; s < P.batch; ++s) f += max(0, __builtin_amdgcn_readlane(g, s) - r_lane);
-                const unsigned long long above = __ballot(f > j);  // F decreases with the level: low lanes
-                if (above == 0) break;
-                const int n = __popcll(above);
-                level = base + n - 1;
-                f_level = __builtin_amdgcn_readlane(f, n - 1);
-                if (n < 64) break;
-            }
+            level = base + n - 1;
+            f_level = __builtin_amdgcn_readlane(f, n - 1);
+            if (n < 64) break;
         }
         if (level < 0) return false;                           // past the last pair
         const unsigned long long owners = __ballot(g > level); // sequences that have this row group
@@ -132,11 +158,11 @@ __device__ __forceinline__ bool locate_row_group(const StaircaseParams& P, int j
         const unsigned long long hit = __ballot(((owners >> lane) & 1ull) != 0 && before == nth);
         b = __ffsll((long long)hit) - 1;
         rg = level;
-        if (b < 0) return false;
-    } else {
-        b = j % P.batch;
-        rg = P.n_row_groups - 1 - j / P.batch;
+        return b >= 0;
     }
+    // more than 64 sequences with more than 64 row groups each: the full (level x sequence) rectangle
+    b = j % P.batch;
+    rg = P.n_row_groups - 1 - j / P.batch;
     return true;
 }
 
@@ -447,8 +473,9 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     P.log2_s = log2_s;
     P.c = scale * kLog2e;
     // dense numbering: at most ceil((L_b + S - 1) / rows) row groups per sequence
-    const int64_t n_pairs = batch <= 64 ? (total_tokens + (int64_t)batch * (staircase_size + rows_per_wg - 2)) / rows_per_wg
-                                        : (int64_t)P.n_row_groups * batch;
+    const bool dense = batch <= 64 || (P.n_row_groups <= 64 && batch <= kDenseMaxBatch);
+    const int64_t n_pairs = dense ? (total_tokens + (int64_t)batch * (staircase_size + rows_per_wg - 2)) / rows_per_wg
+                                  : (int64_t)P.n_row_groups * batch;
     // Two query heads per wavefront when the heads of a KV head pair up and 32-bit row offsets suffice.
     const int64_t row_elems = k_stride_t > v_stride_t ? k_stride_t : v_stride_t;
     // Sequences of a few hundred tokens are left to the one-head kernel: a pair workgroup owns a whole CU and its fixed cost (set-up,

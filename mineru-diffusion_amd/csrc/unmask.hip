@@ -398,8 +398,12 @@ __global__ __launch_bounds__(kThreads) void confidence_argmax_kernel(
                 for (int i = 0; i < EPC; ++i) offer(x[i], c0 + i, rn.at(c0 + i));
             }
             if (NOISE == 2) {
-                // the wavefront's best so far, to everybody (only when it has grown: few chunks of a row raise it)
-                if (__builtin_amdgcn_ballot_w64(best > seen) != 0) {
+                // the wavefront's best so far, to everybody (only when it has grown: few chunks of a row raise it).
+                // Only with all 64 lanes still in the loop: on the row's last, partly filled trip the lanes that
+                // have left are switched off, a shuffle reads 0 from them, and a 0 published above a row whose
+                // noisy logits are all negative would let the others skip the real winner.  Not publishing on
+                // that one trip costs nothing (an old lead_seen only makes the skip test more cautious).
+                if (__builtin_amdgcn_ballot_w64(best > seen) != 0 && __builtin_amdgcn_ballot_w64(true) == ~0ull) {
                     float wb = best;
 #pragma unroll
                     for (int off = 32; off >= 1; off >>= 1) wb = fmaxf(wb, __shfl_xor(wb, off));

@@ -69,7 +69,7 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     pa = lambda **kw: L.mdx_paged_block_attn(                                                  # noqa: E731
         one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,
         4, kw.get("sq", 32), 16, 8, kw.get("d", 128), 17, kw.get("page", 256), 100, 0.1, 0, kw.get("ws", null), kw.get("ws_bytes", 0), null)
-    assert pa(sq=33) == -2
+    assert pa(sq=129) == -2 and b"queries per sequence" in L.mdx_last_error()    # up to four tiles of 32 queries
     assert pa(page=100) == -2
     assert pa(d=256) == -2 and b"head_dim" in L.mdx_last_error()
     assert pa(d=40) == -2
@@ -89,7 +89,8 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     sl = lambda counters, nbytes: L.mdx_paged_block_attn_single_launch(                          # noqa: E731
         one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,
         32, 32, 16, 8, 128, 17, 256, 100, 0.1, 0, big, ws32, counters, nbytes, null)
-    assert ws32 > 0 and L.mdx_paged_block_attn_counter_bytes(32, 16, 8) == 32 * 8 * 4
+    # one counter per (sequence, head group, query tile), sized for the longest block (four tiles of 32 queries)
+    assert ws32 > 0 and L.mdx_paged_block_attn_counter_bytes(32, 16, 8) == 32 * 8 * 4 * 4
     assert sl(null, 0) == -3 and b"counters" in L.mdx_last_error()
     assert sl(one, 32 * 8 * 4 - 4) == -3
     assert sl(ctypes.c_void_p(18), 4096) == -3 and b"aligned" in L.mdx_last_error()

@@ -162,6 +162,21 @@ def test_paged_head_layouts_and_short_blocks(dev, hq, hkv, sq):
     _check_paged(dev, [300, 1500], seed=hq + sq, hq=hq, hkv=hkv, sq=sq)
 
 
+@pytest.mark.parametrize("sq", [33, 64, 100, 128])
+@pytest.mark.parametrize("ctxs,hq,hkv", [([300, 1500], 16, 8), ([4128, 0, 64, 2000, 129], 16, 8), ([700] * 33, 16, 8),
+                                         ([2500, 900], 3, 1), ([1800] * 3, 8, 8)])
+def test_paged_blocks_longer_than_32_queries(dev, sq, ctxs, hq, hkv):
+    """Blocks of up to 128 positions (the reference's block length is a configuration field, config.py:48, and
+    sdar_attention.py:50-55 passes whatever [bs, S, Hq, d] it gets): 2 to 4 query tiles per sequence, with split and
+    whole sequences, padding rows, a block length that is not a multiple of 32, odd head ratios; the context
+    includes the block itself, so it is never shorter than the block except for padding rows."""
+    ctxs = [c if c == 0 else max(c, sq) for c in ctxs]
+    o = _check_paged(dev, ctxs, seed=sq + len(ctxs), hq=hq, hkv=hkv, sq=sq, pool=sum((c + 255) // 256 for c in ctxs) + 3)
+    for b, c in enumerate(ctxs):
+        if c == 0:
+            assert o[b].abs().sum().item() == 0
+
+
 def test_paged_page_sizes(dev):
     _check_paged(dev, [900, 130], seed=9, page=128, pool=32)
     _check_paged(dev, [900, 130], seed=10, page=512, pool=8)
@@ -349,7 +364,7 @@ def test_attention_with_uniformly_low_and_constant_scores(dev):
 
 
 def test_prefill_many_short_sequences(dev):
-    """More than 64 sequences (rectangular launch grid instead of the dense numbering), exactly 64,
+    """More than 64 sequences (the lookup walks them 64 at a time), exactly 64,
     lengths from 0 to a few blocks, block sizes below and above the 32 rows of a wavefront."""
     g = torch.Generator().manual_seed(51)
     for B, S in ((150, 32), (64, 32), (90, 4), (70, 128)):
@@ -357,6 +372,23 @@ def test_prefill_many_short_sequences(dev):
         lens[0], lens[5], lens[-1] = 1, 0, 139
         _check_prefill(dev, lens, S, hq=4, hkv=2, seed=B + S)
         _check_prefill(dev, lens[:7], S, hq=3, hkv=1, seed=B)          # odd head ratio: the one-head kernel
+
+
+@pytest.mark.parametrize("B,lo,hi,hq,hkv", [(200, 0, 700, 4, 2), (512, 0, 200, 4, 2), (65, 500, 900, 16, 8), (129, 100, 640, 3, 1)])
+def test_prefill_hundreds_of_sequences_are_numbered_densely(dev, B, lo, hi, hq, hkv):
+    """The reference's scheduler admits up to 512 sequences per prefill (config.py:38, scheduler.py:24-44): launches of
+    more than 64 sequences keep the dense, heaviest-first workgroup numbering (64 sequences per step of the lookup)
+    as long as no sequence exceeds 64 row groups; pair kernel and one-head kernel, empty sequences included."""
+    g = torch.Generator().manual_seed(B + hi)
+    lens = [int(x) for x in torch.randint(lo, hi + 1, (B,), generator=g)]
+    lens[3], lens[-1], lens[B // 2] = 0, hi, 1
+    _check_prefill(dev, lens, 32, hq=hq, hkv=hkv, seed=B)
+
+
+def test_prefill_many_sequences_with_one_beyond_64_row_groups(dev):
+    """More than 64 sequences AND a sequence of more than 64 row groups (8 K tokens): the rectangular grid."""
+    lens = [40] * 70 + [8300] + [130] * 10
+    _check_prefill(dev, lens, 32, hq=4, hkv=2, seed=8300)
 
 
 def test_paged_pair_per_cu_batches(dev):

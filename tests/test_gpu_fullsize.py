@@ -149,3 +149,72 @@ def test_config4_decisions_on_rounding_boundaries(dev):
                 near += 1
     print(f"config-4 boundary flips: {flips} positions in {near} blocks over 8 (threshold, k) settings")
     assert flips == 0
+
+
+def test_config2_real_pool(dev):
+    """bench.py's config-2 input as it is timed: 16 sequences over a 65 536-page pool (2 x 32 GiB; page ids up to
+    65 535, byte offsets up to 32 GiB, far beyond 32-bit element indices), both launch forms of the paged attention.
+    Only the referenced pages (at most 272 per cache) come back to the host, where the oracle runs on a compacted
+    copy of the pool with a renumbered page table; max-abs < 2e-2.  Then store_kvcache into slots whose element
+    offsets lie above 2^31, checked bit for bit with their neighbouring slots."""
+    import bench
+    import mdx
+    c2 = bench.make_cfg2(dev, n_sets=1)
+    bt, lens, q = c2["tables"][0], c2["lens"], c2["q"]
+    kc, vc = c2["k_cache"], c2["v_cache"]
+    assert kc.shape == (65536, PAGE, HKV, D) and bt.shape[0] == 16
+    ids = bt[bt >= 0].long()
+    assert int(ids.max()) > 60000 and ids.numel() <= 272
+    assert int(ids.max()) * PAGE * HKV * D > 2 ** 33                        # element offsets need 64 bits
+    scale = 1 / math.sqrt(D)
+    o_two = mdx.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens, block_table=bt, softmax_scale=scale, counters=False)
+    o_one = mdx.flash_attn_with_kvcache(q, kc, vc, cache_seqlens=lens, block_table=bt, softmax_scale=scale)
+    torch.cuda.synchronize()
+    # compacted pool on the host: page i of the copy = page ids[i] of the real pool
+    remap = {int(p): i for i, p in enumerate(ids.tolist())}
+    hk, hv = kc[ids].cpu(), vc[ids].cpu()
+    hbt = torch.tensor([[remap.get(int(p), -1) for p in row] for row in bt.cpu().tolist()], dtype=torch.int32)
+    ref = oracle.paged_block_attn(q.cpu(), hk, hv, hbt, lens.cpu(), scale)
+    for o in (o_two, o_one):
+        err = (o.float().cpu() - ref).abs().max().item()
+        assert err < 2e-2, err
+    assert torch.equal(o_two, o_one)
+
+    # store into the last pages of the pool: slot * 1024 elements > 2^31 from page 8192 on
+    g = torch.Generator().manual_seed(22)
+    free = sorted(set(range(65000, 65536)) - set(ids.tolist()))[:6]
+    n = 700
+    slots = torch.tensor(oracle.get_slots(free, 100, 100 + n), dtype=torch.int32)
+    slots[::7] = -1
+    assert int(slots.max()) * HKV * D > 2 ** 31
+    key = torch.randn(n, HKV, D, generator=g).bfloat16()
+    fused = torch.randn(n, 4096, generator=g).bfloat16()
+    val = fused[:, 3072:].view(n, HKV, D)                                    # strided rows, as in the engine
+    pages = torch.tensor(free, device=dev)
+    kc[pages] = 0
+    vc[pages] = 0
+    mdx.store_kvcache(key.to(dev), fused.to(dev)[:, 3072:].view(n, HKV, D), kc, vc, slots.to(dev))
+    torch.cuda.synchronize()
+    ek = np.zeros((len(free) * PAGE, HKV * D), dtype=np.int16)
+    ev = np.zeros_like(ek)
+    local = {p: i for i, p in enumerate(free)}
+    lslots = np.array([-1 if s < 0 else local[s // PAGE] * PAGE + s % PAGE for s in slots.tolist()], dtype=np.int32)
+    oracle.store_kvcache(_i16(key), _i16(val), ek, ev, lslots)
+    assert np.array_equal(_i16(kc[pages]).reshape(-1, HKV * D), ek)
+    assert np.array_equal(_i16(vc[pages]).reshape(-1, HKV * D), ev)
+    del c2, kc, vc
+    torch.cuda.empty_cache()
+
+
+def test_config5_full_size_properties(dev):
+    """Config 5 at full size (28 layers, hidden 2048, batch 32, 1088-token prompts, 2048 new tokens in 32-token blocks,
+    8 denoising passes per block) through the engine's device loop, as bench.py times it.  No oracle covers a
+    2-billion-parameter run; what must hold whatever the weights is asserted inside run_cfg5: every sequence
+    complete, no mask token in the output, one step-map entry per token, and exactly 64 x 9 - 1 decode passes (no
+    confidence of a random-init model reaches the threshold, so every denoising pass commits k = 4 positions)."""
+    import bench
+    out = bench.run_cfg5(dev)
+    assert out["committed_tokens"] == 32 * 2048 and out["layers"] == 28 and out["batch"] == 32
+    assert out["decode_passes"] == 64 * 9 - 1 and out["prefill_passes"] >= 1
+    print(f"config 5: {out['tokens_per_s']} tokens/s, {out['ms_per_decode_pass']} ms per decode pass")
+    torch.cuda.empty_cache()

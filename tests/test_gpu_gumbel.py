@@ -113,6 +113,33 @@ def test_seeded_sampling_of_peaked_rows_skips_only_what_cannot_win(dev, dtype):
     assert len(set(x0.flatten().tolist())) > 10
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bs,S,V", [(1, 4, 151936), (2, 8, 50001), (40, 32, 5000), (3, 5, 2048 * 3 + 8 * 70)])
+def test_seeded_sampling_of_rows_whose_noisy_logits_are_all_negative(dev, dtype, bs, S, V):
+    """Rows shifted to about -60, so that every noisy logit is negative, with chunk counts that are not a multiple
+    of the workgroup's width: on the last, partly filled trip of a row the wavefront's lead is not published (a
+    shuffle over switched-off lanes reads 0, which would beat every real value here and let the other wavefronts
+    skip the winner).  Picks must be those of the tensor-noise path, which skips nothing."""
+    import mdx
+    g = torch.Generator().manual_seed(V)
+    logits = (torch.randn(bs, S, V, generator=g) * 2 - 60)
+    # winners late in the row and inside the last trips of other wavefronts
+    for b in range(bs):
+        for r in range(S):
+            at = V - 1 - int(torch.randint(0, min(V, 4096), (1,), generator=g))
+            logits[b, r, at] += 14.0
+    logits = logits.to(dtype).to(dev)
+    temps = torch.linspace(0.7, 1.4, bs, device=dev)
+    for offset in range(4):
+        x0, p = mdx.confidence_argmax(logits, temps, seed=21, offset=offset)
+        noise = mdx.gumbel_noise(bs * S, V, 21, offset, device=dev)
+        x0n, pn = mdx.confidence_argmax(logits, temps, noise=noise.view(bs, S, V))
+        torch.cuda.synchronize()
+        assert torch.equal(x0, x0n)
+        torch.testing.assert_close(p, pn, rtol=3e-6, atol=0)
+        assert float(((logits.float() / temps.view(-1, 1, 1)) + noise.view(bs, S, V)).max()) < 0
+
+
 def test_seeded_unmask_step_equals_the_step_with_the_noise_tensor(dev):
     import mdx
     g = torch.Generator().manual_seed(3)
