@@ -239,3 +239,46 @@ def test_transfer_schedule_helper_matches_the_oracle():
         assert sum(got) == block and max(got) - min(got) <= 1 and got == sorted(got, reverse=True)
     assert mdx.num_transfer_tokens(3, 8) == [1, 1, 1, 0, 0, 0, 0, 0]
 
+
+
+def test_oracle_block_advance_against_a_hand_written_trace():
+    """One lane, a block of 4 positions, budget of one block, written out by hand from layers/sampler.py:56-59 and
+    engine/scheduler.py:65-82 (no engine code involved).  Pass 0 commits positions 2 and 0, pass 1 commits 1 and 3
+    and thereby ends the denoising (phase -> caching), pass 2 is the caching pass: the block is appended, the
+    length grows by 4, the budget is spent (phase -> idle), the lane's tokens become a fresh all-mask block."""
+    M = MASK
+    tokens = np.array([[M, M, M, M]], dtype=np.int64)
+    step_map = np.zeros((1, 4), dtype=np.int32)
+    step, phase, lens = np.array([0], dtype=np.int32), np.array([1]), np.array([10])
+    first, budget, stop = np.array([10]), np.array([4]), np.full((1, 4), -1)
+
+    # pass 0: the sampler wrote tokens 7 and 5 at positions 2 and 0
+    tokens[0, 2], tokens[0, 0] = 7, 5
+    transfer = np.array([[True, False, True, False]])
+    tokens, step_map, step, phase, lens, appended, status = oracle.block_advance(
+        tokens, transfer, step_map, step, phase, lens, first, budget, stop, M)
+    assert tokens.tolist() == [[5, M, 7, M]] and step_map.tolist() == [[0, 0, 0, 0]]     # committed at step 0
+    assert step.tolist() == [1] and phase.tolist() == [1] and lens.tolist() == [10] and appended == [None]
+    assert status == [(1, 10, 2, 2)]                                                    # denoising, 2 masked left, 2 committed
+
+    # pass 1: positions 1 and 3 get 8 and 9: nothing masked is left, the next pass only caches
+    tokens[0, 1], tokens[0, 3] = 8, 9
+    transfer = np.array([[False, True, False, True]])
+    tokens, step_map, step, phase, lens, appended, status = oracle.block_advance(
+        tokens, transfer, step_map, step, phase, lens, first, budget, stop, M)
+    assert tokens.tolist() == [[5, 8, 7, 9]] and step_map.tolist() == [[0, 1, 0, 1]]
+    assert step.tolist() == [2] and phase.tolist() == [2] and lens.tolist() == [10] and appended == [None]
+    assert status == [(2, 10, 0, 2)]
+
+    # pass 2 (caching): nothing is committed; the block is appended and the budget of 4 new tokens is spent
+    transfer = np.zeros((1, 4), dtype=bool)
+    tokens, step_map, step, phase, lens, appended, status = oracle.block_advance(
+        tokens, transfer, step_map, step, phase, lens, first, budget, stop, M)
+    assert appended[0][0].tolist() == [5, 8, 7, 9] and appended[0][1].tolist() == [0, 1, 0, 1]
+    assert tokens.tolist() == [[M, M, M, M]] and lens.tolist() == [14] and phase.tolist() == [0] and step.tolist() == [3]
+    assert status == [(0, 14, 0, 0)]
+
+    # the same lane with a budget of two blocks goes back to denoising instead, with 4 masked positions
+    t2, _, _, p2, l2, _, s2 = oracle.block_advance(np.array([[5, 8, 7, 9]]), transfer, np.array([[0, 1, 0, 1]], dtype=np.int32),
+                                                   np.array([2], dtype=np.int32), np.array([2]), np.array([10]), first, np.array([8]), stop, M)
+    assert p2.tolist() == [1] and l2.tolist() == [14] and s2 == [(1, 14, 4, 0)] and t2.tolist() == [[M, M, M, M]]
