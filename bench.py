@@ -274,7 +274,7 @@ def make_cfg4(dev, n_sets=2, seed=4):
 
 
 # ----------------------------------------------------------------------------- config 5
-def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, masked_rows_only=True, gumbel_seed=None):
+def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, masked_rows_only=True, gumbel_seed=None, fused_head=True):
     """Random-init SDAR-shaped decoder (28 layers, hidden 2048, Hq 16 / Hkv 8 / d 128, SwiGLU 6144,
     vocab 151936), batch 32, 1024 random prefix embeddings + 64 prompt tokens per sequence, 2048 new
     tokens in 32-token blocks, k = 32/8 = 4 committed positions per denoising pass, threshold 0.9.
@@ -285,7 +285,7 @@ def run_cfg5(dev, layers=28, batch=32, new_tokens=2048, steps_per_block=8, maske
     model = Decoder(cfg, dev, seed=5)
     pages_per_seq = (1088 + new_tokens + PAGE - 1) // PAGE + 1
     eng = BlockDiffusionEngine(model, num_pages=batch * pages_per_seq + 8, shuffle_pages_seed=5, decode_graphs=True, max_model_len=4096,
-                               masked_rows_only=masked_rows_only, gumbel_seed=gumbel_seed)
+                               masked_rows_only=masked_rows_only, gumbel_seed=gumbel_seed, fused_head=fused_head)
     g = torch.Generator().manual_seed(5)
     prompts = []
     for _ in range(batch):
@@ -719,6 +719,8 @@ def main():
             decode["with_full_logits"] = {k: full[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass", "vocabulary_projection")}
             noisy = run_cfg5(dev, gumbel_seed=5)
             decode["with_gumbel_sampling"] = {k: noisy[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass")}
+            two = run_cfg5(dev, fused_head=False)
+            decode["with_library_projection_and_separate_confidence_pass"] = {k: two[k] for k in ("tokens_per_s", "seconds", "ms_per_decode_pass")}
 
     # ---------------- CPU baseline (bounded) -------------------------------------------------------------
     cpu = None

@@ -198,6 +198,28 @@ int mdx_paged_block_attn_static(const void* q, void* o, const void* k_cache, con
                                 float scale, int32_t dtype, mdx_stream_t stream);
 
 /*
+ * Vocabulary projection fused with confidence + argmax -- replaces, for rows that are only wanted for
+ * the unmask step, ParallelLMHead.forward's F.linear(x, weight)
+ * (engines/nano_dvlm/nanovllm/layers/embed_head.py:61-67) followed by Sampler.prepare without noise
+ * (layers/sampler.py:11-22); the [rows, vocab] logits are never written.
+ *
+ * x [rows, hidden] and w [vocab, hidden], MDX_BF16, row strides in elements (multiples of 8, 16-byte
+ * aligned bases); hidden a multiple of 128.  The logits x . w^T are accumulated in fp32 and rounded to
+ * bf16, as the projection's output is in the reference; then x0[r] = first index of the row's maximum,
+ * x0_p[r] = softmax(logits / T)[x0[r]].  temperatures (NULL = 1.0): row r uses entry
+ * (row_ids ? row_ids[r] : r) / rows_per_temp, so that rows compacted out of [bs, block] keep their
+ * sequence's temperature; row_ids may be NULL.  The workspace (mdx_lm_head_confidence_workspace_bytes,
+ * 16-byte aligned, contents need no initialisation) holds one 16-byte record per row and 128-entry slice
+ * of the vocabulary.  Two launches: the projection tiles, then one wavefront per row folding its records.
+ */
+int64_t mdx_lm_head_confidence_workspace_bytes(int64_t rows, int64_t vocab);
+int mdx_lm_head_confidence(const void* x, int64_t x_row_stride, const void* w, int64_t w_row_stride,
+                           const float* temperatures, int32_t rows_per_temp, const int64_t* row_ids,
+                           int64_t* x0, float* x0_p,
+                           int64_t rows, int64_t vocab, int64_t hidden,
+                           void* workspace, int64_t workspace_bytes, mdx_stream_t stream);
+
+/*
  * Confidence + argmax over the vocabulary -- replaces Sampler.prepare
  * (engines/nano_dvlm/nanovllm/layers/sampler.py:11-22).
  *

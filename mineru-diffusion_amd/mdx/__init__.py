@@ -21,7 +21,7 @@ without the built library or on a non-GPU tensor raises.
 from .context import Context, get_context, set_context, reset_context  # noqa: F401
 from .ops import (  # noqa: F401
     sparse_attn_varlen, sparse_attn_varlen_v2, store_kvcache, store_kvcache_maybe4d,
-    flash_attn_with_kvcache, confidence_argmax, gumbel_noise, filter_logits, num_transfer_tokens, select_transfer, unmask_step, qk_norm_rope_store, rms_norm, silu_and_mul,
+    flash_attn_with_kvcache, confidence_argmax, lm_head_confidence, gumbel_noise, filter_logits, num_transfer_tokens, select_transfer, unmask_step, qk_norm_rope_store, rms_norm, silu_and_mul,
 )
 from .layers import Attention, Sampler  # noqa: F401
 from ._lib import lib, library_path, MdxError  # noqa: F401

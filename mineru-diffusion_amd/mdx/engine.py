@@ -32,7 +32,7 @@ from torch import nn
 from . import _lib
 from .context import get_context, reset_context, set_context
 from .layers import Attention
-from .ops import (confidence_argmax, flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
+from .ops import (confidence_argmax, lm_head_confidence, flash_attn_with_kvcache, qk_norm_rope_store, rms_norm, select_transfer, silu_and_mul,
                   sparse_attn_varlen, unmask_step)
 
 PAGE = 256                      # tokens per KV page (Sequence.kvcache_block_size, sequence.py:17)
@@ -325,8 +325,11 @@ class BlockDiffusionEngine:
     def __init__(self, model: Decoder, num_pages: int, max_num_batched_tokens: int = 1 << 20,
                  max_num_seqs: int = 512, shuffle_pages_seed: int | None = None, on_logits=None, unmask=None,
                  decode_graphs: bool = False, max_model_len: int = 8192, masked_rows_only: bool = True,
-                 replay_ahead: bool = True, gumbel_seed: int | None = None):
+                 replay_ahead: bool = True, gumbel_seed: int | None = None, fused_head: bool = True,
+                 fused_head_min_rows: int = 384):
         self.model = model
+        # device loop: vocabulary projection + confidence in one pass without logits in HBM, from this many rows on
+        self.fused_head, self.fused_head_min_rows = fused_head, fused_head_min_rows
         self.decode_graphs = decode_graphs                 # decode through the device loop (HIP graphs per batch size)
         self.max_model_len = max_model_len
         # Gumbel noise on the scaled logits before the argmax, as Sampler.prepare draws it (sampler.py:15-18);
@@ -613,15 +616,28 @@ class BlockDiffusionEngine:
             stream = torch.cuda.current_stream(self.device).cuda_stream
             _lib.check(_lib.lib().mdx_masked_rows(g["ids"].data_ptr(), g["phase"].data_ptr(), self.c.mask_token_id, gbs, S,
                                                   rows.data_ptr(), cap, g["n_rows"].data_ptr(), stream), "masked_rows")
-            logits = F.linear(flat.index_select(0, rows), self.model.lm_head)
-            x0, p = confidence_argmax(logits, g["temps"].index_select(0, rows // S), **self._draw(g, rows))
+            if self._fused_head(cap):
+                x0, p = lm_head_confidence(flat.index_select(0, rows), self.model.lm_head, g["temps"], rows_per_temp=S, row_ids=rows)
+            else:
+                logits = F.linear(flat.index_select(0, rows), self.model.lm_head)
+                x0, p = confidence_argmax(logits, g["temps"].index_select(0, rows // S), **self._draw(g, rows))
             g["x0"].index_copy_(0, rows, x0)
             g["x0_p"].index_copy_(0, rows, p)
         else:
-            logits = F.linear(flat, self.model.lm_head).view(gbs, S, -1)
-            x0, p = confidence_argmax(logits, g["temps"], **self._draw(g, None))
+            if self._fused_head(cap):
+                x0, p = lm_head_confidence(flat, self.model.lm_head, g["temps"], rows_per_temp=S)
+            else:
+                logits = F.linear(flat, self.model.lm_head).view(gbs, S, -1)
+                x0, p = confidence_argmax(logits, g["temps"], **self._draw(g, None))
             g["x0"].copy_(x0.view(-1))
             g["x0_p"].copy_(p.view(-1))
+
+    def _fused_head(self, rows: int) -> bool:
+        """Projection and confidence in one pass that never writes the logits (mdx_lm_head_confidence): taken where it
+        is the faster of the two (from a few hundred rows on; below that the library GEMM + the vocabulary pass
+        win), for bf16 weights without sampling noise."""
+        return (self.fused_head and self.gumbel_seed is None and rows >= self.fused_head_min_rows
+                and self.model.lm_head.dtype == torch.bfloat16 and self.model.lm_head.shape[1] % 128 == 0)
 
     def _draw(self, g, rows):
         """Generator arguments of a device-loop pass: the lanes' own pass counter as the offset, and for compacted

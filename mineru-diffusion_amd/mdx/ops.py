@@ -325,6 +325,44 @@ def confidence_argmax(logits: torch.Tensor, temperatures: torch.Tensor | None = 
     return x0.view(lead), x0_p.view(lead)
 
 
+def lm_head_confidence(x: torch.Tensor, weight: torch.Tensor, temperatures: torch.Tensor | None = None,
+                       rows_per_temp: int | None = None, row_ids: torch.Tensor | None = None):
+    """ParallelLMHead.forward's F.linear(x, weight) (nanovllm/layers/embed_head.py:61-67) followed by
+    Sampler.prepare without noise (layers/sampler.py:11-22), in one pass that never writes the logits:
+    x [..., hidden] bf16, weight [vocab, hidden] bf16 -> (x0 int64 [...], x0_p fp32 [...]) = argmax and softmax
+    confidence of bf16(x . weight^T) / T.  temperatures [n] fp32: row r uses entry (row_ids[r] if given else r)
+    // rows_per_temp (default rows / n), so that compacted rows keep the temperature of their sequence."""
+    _need_gpu(x, weight, temperatures, row_ids)
+    assert x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "lm_head_confidence: bf16 only"
+    lead = x.shape[:-1]
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    assert weight.dim() == 2 and weight.stride(-1) == 1 and weight.shape[1] == x2.shape[1]
+    rows, hidden = x2.shape
+    vocab = weight.shape[0]
+    t_ptr, rpt = None, 1
+    if temperatures is not None:
+        temperatures = temperatures.reshape(-1).to(torch.float32).contiguous()
+        if rows_per_temp is None:
+            assert rows % temperatures.numel() == 0
+            rows_per_temp = rows // temperatures.numel()
+        t_ptr, rpt = temperatures.data_ptr(), int(rows_per_temp)
+    ids_ptr = None
+    if row_ids is not None:
+        assert row_ids.dtype == torch.int64 and row_ids.is_contiguous() and row_ids.numel() >= rows
+        ids_ptr = row_ids.data_ptr()
+    x0 = torch.empty(rows, dtype=torch.int64, device=x.device)
+    x0_p = torch.empty(rows, dtype=torch.float32, device=x.device)
+    L = _lib.lib()
+    ws_bytes = L.mdx_lm_head_confidence_workspace_bytes(rows, vocab)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
+    rc = L.mdx_lm_head_confidence(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), t_ptr, rpt, ids_ptr,
+                                  x0.data_ptr(), x0_p.data_ptr(), rows, vocab, hidden, ws.data_ptr(), ws_bytes, _stream(x))
+    check(rc, "lm_head_confidence")
+    return x0.view(lead), x0_p.view(lead)
+
+
 def filter_logits(logits: torch.Tensor, top_k: int = 0, top_p: float = 1.0,
                   temperatures: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
     """top_k_logits then top_p_logits of the HF variant (modeling_mineru_diffusion.py:585-600, in the

@@ -196,6 +196,32 @@ def test_masked_rows_only_sampling_matches_full_logits(dev, temps):
         assert sum(int(a == b) for a, b in zip(ma, mb)) >= 90
 
 
+@pytest.mark.parametrize("rows_only", [False, True])
+@pytest.mark.parametrize("temps", [(1.0, 1.0, 1.0), (1.0, 0.7, 1.3)])
+def test_fused_head_generates_like_projection_plus_confidence_pass(dev, temps, rows_only):
+    """The device loop with the vocabulary projection fused into the confidence reduction (no logits in memory,
+    mdx_lm_head_confidence; forced on for this small batch) against the same engine on the library GEMM + the
+    vocabulary pass: same pass count, same committed tokens and step maps up to near-ties (the two sum the
+    products in different orders, which can move a logit to the neighbouring bf16 value)."""
+    from mdx.engine import BlockDiffusionEngine, SamplingParams
+    cfg, model = _tiny(dev)
+    outs = []
+    for fused in (False, True):
+        eng = BlockDiffusionEngine(model, num_pages=16, shuffle_pages_seed=3, decode_graphs=True, max_model_len=1024,
+                                   masked_rows_only=rows_only, fused_head=fused, fused_head_min_rows=1)
+        g = torch.Generator().manual_seed(2)
+        seqs = [eng.add_request(torch.randint(0, 900, (n,), generator=g).tolist(),
+                                SamplingParams(max_new_tokens=96, ignore_eos=True, transfer_count=4, temperature=t))
+                for n, t in zip((290, 33, 150), temps)]
+        eng.generate()
+        outs.append([(s.completion_token_ids, list(s.step_map)) for s in seqs])
+        assert eng.stats["decode_passes"] == 3 * 9 - 1
+    for (ta, ma), (tb, mb) in zip(*outs):
+        assert len(ta) == len(tb) == 96 and cfg.mask_token_id not in tb
+        assert sum(int(a == b) for a, b in zip(ta, tb)) >= 90
+        assert sum(int(a == b) for a, b in zip(ma, mb)) >= 90
+
+
 def test_replay_ahead_changes_nothing(dev):
     """Enqueuing the next decode forward before the host bookkeeping of the current pass is pure
     scheduling: same tokens, same step maps, same pass count, with a request that arrives late
