@@ -457,7 +457,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-full-logits-leg", action="store_true",
                     help="decode leg: skip the second generation that projects all 32 positions of every block")
-    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,decode (default all; gumbel and filter run inside unmask), plus power (only when named: socket power and clock under the attention kernel and the library GEMM)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,lmhead,decode (default all; gumbel and filter run inside unmask), plus power (only when named: socket power and clock under the attention kernel and the library GEMM)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -705,6 +705,50 @@ def main():
                                                         note="off by default in the reference; with both filters on a row is read five times (four counting passes and the writing pass)"))
             del flt_out
         del c4
+        torch.cuda.empty_cache()
+
+    # ---------------- vocabulary projection fused with the confidence reduction ------------------------------
+    if want("lmhead"):
+        # config 5's head: [rows, 2048] x [151936, 2048]^T at the row counts the decode loop projects (eighths of the
+        # 1024 positions of a pass); fused (no logits in memory) against the library GEMM + the vocabulary pass
+        L = mdx.lib()
+        hid = 2048
+        gh = torch.Generator(device=dev).manual_seed(6)
+        w_head = (torch.randn(VOCAB, hid, generator=gh, device=dev) * 0.02).bfloat16()
+        head = {}
+        for rows_h in (1024, 512, 256):
+            xh = torch.randn(rows_h, hid, generator=gh, device=dev).bfloat16()
+            x0h = torch.empty(rows_h, dtype=torch.int64, device=dev)
+            ph = torch.empty(rows_h, dtype=torch.float32, device=dev)
+            wsb = L.mdx_lm_head_confidence_workspace_bytes(rows_h, VOCAB)
+            wsh = torch.empty(wsb, dtype=torch.uint8, device=dev)
+            lg = torch.empty(rows_h, VOCAB, dtype=torch.bfloat16, device=dev)
+            wsb2 = L.mdx_confidence_argmax_workspace_bytes(rows_h, VOCAB)
+            ws2h = torch.empty(max(wsb2, 16), dtype=torch.uint8, device=dev)
+            x0t = torch.empty_like(x0h)
+            pt = torch.empty_like(ph)
+
+            def fused(i):
+                rc = L.mdx_lm_head_confidence(xh.data_ptr(), xh.stride(0), w_head.data_ptr(), w_head.stride(0), None, 1, None,
+                                              x0h.data_ptr(), ph.data_ptr(), rows_h, VOCAB, hid, wsh.data_ptr(), wsb, raw_stream())
+                assert rc == 0
+
+            def two_step(i):
+                torch.matmul(xh, w_head.t(), out=lg)
+                rc = L.mdx_confidence_argmax(lg.data_ptr(), VOCAB, 0, None, 1, None, 0, x0t.data_ptr(), pt.data_ptr(), rows_h, VOCAB,
+                                             ws2h.data_ptr(), wsb2, raw_stream())
+                assert rc == 0
+            f_ms, f_min = time_kernel(fused, 20 + W, max(5, K // 2), graph=True)
+            t_ms, _ = time_kernel(two_step, 20 + W, max(5, K // 2), graph=True)
+            flops_h = 2 * rows_h * VOCAB * hid
+            e = op_entry(f_ms, f_min, "mfma", flops_h, 1e9, PEAK_MFMA_TFLOPS, "TFLOP/s",
+                         dict(rows=rows_h, library_gemm_plus_confidence_pass_ms=round(t_ms, 4),
+                              same_tokens=round(float((x0h == x0t).float().mean()), 4)))
+            head[f"rows_{rows_h}"] = e
+            if rows_h == 1024:
+                result_ops["lm_head_confidence"] = e
+        result_ops["lm_head_confidence"]["other_row_counts"] = {k: v for k, v in head.items() if k != "rows_1024"}
+        del w_head
         torch.cuda.empty_cache()
 
     # ---------------- config 5: end-to-end block-diffusion decode ---------------------------------------

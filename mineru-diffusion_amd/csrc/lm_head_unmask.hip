@@ -122,10 +122,18 @@ __global__ __launch_bounds__(kThreads) void lm_head_finalize_kernel(const LmHead
         idx = (m2 > m) ? i2 : ((m2 == m) ? min(idx, i2) : idx);
         m = M;
     };
-    const Record* rec = P.records + (int64_t)row * P.n_slices;
-    for (int i = lane; i < P.n_slices; i += 64) {
-        const Record q = rec[i];
-        fold(q.m, q.s, q.idx);
+    // the row's records, eight per lane in flight at a time (a fold per load would make this a chain of memory latencies)
+    const u32x4* rec = reinterpret_cast<const u32x4*>(P.records + (int64_t)row * P.n_slices);
+    for (int i0 = lane; i0 < P.n_slices; i0 += 64 * 8) {
+        u32x4 q[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = i0 + 64 * k;
+            q[k] = __builtin_nontemporal_load(rec + (i < P.n_slices ? i : lane));   // (lane < n_slices here: i0 = lane is)
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (i0 + 64 * k < P.n_slices) fold(__uint_as_float(q[k].x), __uint_as_float(q[k].y), (int)q[k].z);
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
