@@ -561,10 +561,35 @@ def main():
             a_r = torch.randn(8192, 8192, device=dev).bfloat16()
             a_z = torch.zeros(8192, 8192, device=dev, dtype=torch.bfloat16)
             gemm_flops = 2 * 8192 ** 3
+            # the matrix pipe alone: register-only loops of back-to-back MFMAs (two wavefronts per SIMD) on N(0,1) bf16
+            # operands -- no kernel that feeds such data through these instructions can run faster under the power limit
+            Lc = mdx.lib()
+            pb, pit = 512, 1600
+            p_ops = torch.randn(pb * 256 * 128, device=dev).bfloat16().view(torch.int16)
+            p_out = torch.empty(pb * 256, device=dev)
+
+            def mfma_loop(shape):
+                rc = Lc.mdx_calib_mfma_loop(shape, p_ops.data_ptr(), p_out.data_ptr(), pb, pit, raw_stream())
+                assert rc == 0
+            # the fused vocabulary projection at 1024 rows (config 5's head), the library's GEMM structure without a softmax
+            hw = (torch.randn(VOCAB, 2048, device=dev) * 0.02).bfloat16()
+            hx = torch.randn(1024, 2048, device=dev).bfloat16()
+            h0 = torch.empty(1024, dtype=torch.int64, device=dev)
+            hp = torch.empty(1024, dtype=torch.float32, device=dev)
+            hws_b = Lc.mdx_lm_head_confidence_workspace_bytes(1024, VOCAB)
+            hws = torch.empty(hws_b, dtype=torch.uint8, device=dev)
+
+            def head_fused():
+                rc = Lc.mdx_lm_head_confidence(hx.data_ptr(), 2048, hw.data_ptr(), 2048, None, 1, None, h0.data_ptr(), hp.data_ptr(),
+                                               1024, VOCAB, 2048, hws.data_ptr(), hws_b, raw_stream())
+                assert rc == 0
             for name, fn, flops in (("staircase_attn_config3_random", lambda: attn_only(0), work3["flops"]),
+                                    ("lm_head_confidence_1024_rows", head_fused, 2 * 1024 * VOCAB * 2048),
                                     ("staircase_attn_config3_zeros", lambda: attn_only(0, z), work3["flops"]),
                                     ("library_gemm_bf16_8192_random", lambda: torch.matmul(a_r, a_r), gemm_flops),
-                                    ("library_gemm_bf16_8192_zeros", lambda: torch.matmul(a_z, a_z), gemm_flops)):
+                                    ("library_gemm_bf16_8192_zeros", lambda: torch.matmul(a_z, a_z), gemm_flops),
+                                    ("mfma_32x32x16_register_loop_random", lambda: mfma_loop(32), Lc.mdx_calib_mfma_loop_flops(32, pb, pit)),
+                                    ("mfma_16x16x32_register_loop_random", lambda: mfma_loop(16), Lc.mdx_calib_mfma_loop_flops(16, pb, pit))):
                 for _ in range(3):
                     fn()
                 torch.cuda.synchronize()
@@ -583,7 +608,7 @@ def main():
                 log(f"[bench] power leg {name}: {stats}")
                 del gr
                 time.sleep(0.5)
-            del zf, z, a_r, a_z
+            del zf, z, a_r, a_z, p_ops, p_out, hw, hx, hws
             torch.cuda.empty_cache()
     if want("store"):
         # three rotating (source, cache) sets, about 900 MB touched per round trip, so the 256 MB

@@ -437,6 +437,16 @@ int mdx_block_advance(int64_t* tokens, const uint8_t* transfer,
                       int32_t* status, int64_t mask_token_id,
                       int32_t bs, int32_t block_len, mdx_stream_t stream);
 
+/*
+ * Calibration helper of bench.py -- no counterpart in the reference.  A register-only loop of back-to-back bf16
+ * MFMAs (shape 32 = v_mfma_f32_32x32x16_bf16, 16 = v_mfma_f32_16x16x32_bf16) in `blocks` workgroups of four
+ * wavefronts, `iters` (rounded up to a multiple of 8) x 8 (x 16) instructions per wavefront, on operands read once:
+ * 64 uint32 per thread (blocks x 256 threads) holding bf16 pairs.  out: one float per thread.  What the matrix pipe
+ * sustains on that data under the board's power limit; mdx_calib_mfma_loop_flops gives the flops of a launch.
+ */
+int64_t mdx_calib_mfma_loop_flops(int32_t shape, int32_t blocks, int32_t iters);
+int mdx_calib_mfma_loop(int32_t shape, const void* operands, float* out, int32_t blocks, int32_t iters, mdx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -143,7 +143,7 @@ def kstep(stage, ks, with_dma, read_next):
         if dma:
             out += dma[m][0]
         out.append(f"{MFMA} {acc(vt, xt)}, {frag(half, vt)}, {frag(half, 4 + xt)}, {acc(vt, xt)}")
-        if read_next and m % 2 == 1:
+        if read_next and m < 8:                            # early in the step: the last of them has half a step to land
             out.append(read_op(nstage, nks, 1 - half, READ_ORDER[issued_new]))
             issued_new += 1
             bound += 1

@@ -50,6 +50,8 @@ SIGNATURES = {
     "mdx_filter_logits": (c_int32, [_P, _I64, _I32, _P, _I32, _I32, _F, _P, _I64, _I64, _I64, _P]),
     "mdx_lm_head_confidence_workspace_bytes": (c_int64, [_I64, _I64]),
     "mdx_lm_head_confidence": (c_int32, [_P, _I64, _P, _I64, _P, _I32, _P, _P, _P, _I64, _I64, _I64, _P, _I64, _P]),
+    "mdx_calib_mfma_loop_flops": (c_int64, [_I32, _I32, _I32]),
+    "mdx_calib_mfma_loop": (c_int32, [_I32, _P, _P, _I32, _I32, _P]),
     "mdx_unmask_step": (c_int32, [_P, _I64, _I32, _P, _P, _I64, _P, _I64, _F, _I32, _P, _P, _P, _P,
                                   _I32, _I32, _I64, _P, _I64, _P]),
 }
