@@ -26,6 +26,14 @@ def bits(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
 
+ONLY = set(sys.argv[1:])          # python tests/golden/make_golden.py [name.npz ...]: write only these (default: all)
+
+
+def save(name, **arrays):
+    if not ONLY or name in ONLY:
+        np.savez_compressed(OUT / name, **arrays)
+
+
 def main():
     g = torch.Generator().manual_seed(20240607)
     d = 128
@@ -38,7 +46,7 @@ def main():
     v = torch.randn(N, hkv, d, generator=g).bfloat16()
     cu = [0, lens[0], N]
     o = oracle.staircase_attn_varlen(q, k, v, cu, S)
-    np.savez_compressed(OUT / "staircase_attn.npz", q=bits(q), k=bits(k), v=bits(v), cu=np.array(cu, np.int32),
+    save("staircase_attn.npz", q=bits(q), k=bits(k), v=bits(v), cu=np.array(cu, np.int32),
                         block=np.int32(S), o=o.float().numpy().astype(np.float32))
 
     # ---- paged single-block attention: contexts of 1, 40 and 270 keys, pages of 32, one padding row
@@ -57,7 +65,7 @@ def main():
         at += n
     lens_t = torch.tensor(ctxs, dtype=torch.int32)
     od = oracle.paged_block_attn(qd, kc, vc, bt, lens_t, 1 / math.sqrt(d))
-    np.savez_compressed(OUT / "paged_block_attn.npz", q=bits(qd), k_cache=bits(kc), v_cache=bits(vc), block_table=bt.numpy(),
+    save("paged_block_attn.npz", q=bits(qd), k_cache=bits(kc), v_cache=bits(vc), block_table=bt.numpy(),
                         context_lens=lens_t.numpy(), o=od.float().numpy().astype(np.float32))
 
     # ---- store_kvcache: 9 tokens into 3 pages of 8 slots, two skipped, V a strided view of a fused projection
@@ -70,7 +78,7 @@ def main():
     vcache = bits(torch.randn(pages, page_len, hkv, d, generator=g).bfloat16())
     k_after, v_after = kcache.copy(), vcache.copy()
     oracle.store_kvcache(key, val, k_after, v_after, slot)
-    np.savez_compressed(OUT / "store_kvcache.npz", fused=bits(fused), slot_mapping=slot, k_cache=kcache, v_cache=vcache,
+    save("store_kvcache.npz", fused=bits(fused), slot_mapping=slot, k_cache=kcache, v_cache=vcache,
                         k_after=k_after, v_after=v_after, hkv=np.int32(hkv))
 
     # ---- unmask step: 3 sequences x 32 positions x 1000 logits; one sequence has peaked rows so that
@@ -89,7 +97,7 @@ def main():
     for b in range(bs):
         c = np.sort(conf[b][conf[b] >= 0])[::-1]
         assert np.all(np.abs(c - 0.9) > 1e-3) and (len(c) <= 4 or c[3] - c[4] > 1e-4), "fixture sits on a tie: change the seed"
-    np.savez_compressed(OUT / "unmask_step.npz", logits=bits(logits), tokens=tokens.numpy(), temperatures=temps,
+    save("unmask_step.npz", logits=bits(logits), tokens=tokens.numpy(), temperatures=temps,
                         mask_id=np.int64(mask_id), threshold=np.float32(0.9), k=np.int32(4),
                         x0=x0.astype(np.int64), x0_p=x0_p.astype(np.float32), tokens_after=after.astype(np.int64),
                         transfer=transfer.astype(np.uint8), count=transfer.sum(-1).astype(np.int32))
@@ -101,7 +109,7 @@ def main():
     y, nr = oracle.add_rms_norm(x, r, w, 1e-6)
     y0, _ = oracle.add_rms_norm(x, None, w, 1e-6)
     gu = (torch.randn(5, 128, generator=g) * 4).bfloat16()
-    np.savez_compressed(OUT / "layer_ops.npz", x=bits(x), residual=bits(r), weight=bits(w), eps=np.float32(1e-6),
+    save("layer_ops.npz", x=bits(x), residual=bits(r), weight=bits(w), eps=np.float32(1e-6),
                         normed=bits(y), new_residual=bits(nr), normed_no_residual=bits(y0),
                         gate_up=bits(gu), act=bits(oracle.silu_and_mul(gu)))
     # ---- sampling: top-k 20 then top-p 0.8 on 8 rows of 600 logits, then the step's Gumbel draw from (seed, offset);
@@ -124,7 +132,7 @@ def main():
     noisy = np.where(np.isfinite(filt), (filt.astype(np.float32) / T8[:, None].astype(np.float32)).astype(np.float64) + noise, -np.inf)
     top2 = np.sort(noisy, axis=-1)[:, -2:]
     assert np.all(top2[:, 1] - top2[:, 0] > 1e-3), "fixture sits on a tie of the noisy argmax: change the seed"
-    np.savez_compressed(OUT / "sampling.npz", logits=bits(lg), temperatures=t2, top_k=np.int32(20), top_p=np.float32(0.8),
+    save("sampling.npz", logits=bits(lg), temperatures=t2, top_k=np.int32(20), top_p=np.float32(0.8),
                         kept=np.isfinite(filt).astype(np.uint8), seed=np.uint64(seed), offset=np.uint64(offset),
                         noise=noise.astype(np.float32), x0=sx0.astype(np.int64), x0_p=sp.astype(np.float32))
 
@@ -160,7 +168,7 @@ def main():
             at = int(lens5[b] - first5[b])
             out_tok[b, at:at + S8], out_step[b, at:at + S8] = ap
     st = np.array([[s[0], lens5[b] if s[1] is None else s[1], s[2], s[3]] for b, s in enumerate(status)], dtype=np.int32)
-    np.savez_compressed(OUT / "block_state.npz", lens=lens5, phase=phase5, block_table=bt5, page=np.int32(page16), block_len=np.int32(S8),
+    save("block_state.npz", lens=lens5, phase=phase5, block_table=bt5, page=np.int32(page16), block_len=np.int32(S8),
                         positions=pos5, slot_mapping=slots5, context_lens=ctx5, mask_id=np.int64(mask_id2),
                         tokens=tok5, rows=rows5, n_rows=np.int32(n5), tokens_selected=tok_sel, transfer=transfer5,
                         step_map=step_map5, step=step5, first_len=first5, max_new=maxnew5, stop_ids=stop5,
@@ -169,6 +177,21 @@ def main():
     for f in sorted(OUT.glob("*.npz")):
         print(f.name, f.stat().st_size, "bytes")
 
+
+    # ---- vocabulary projection fused with the confidence reduction: operands whose products are exact in fp32 in any
+    # order of summation (small integers), so that the logits -- and their bf16 rounding -- are the same numbers for every
+    # implementation; a forced tie between two columns (first index wins), temperatures per group of 8 rows
+    gh = torch.Generator().manual_seed(20240608)
+    rows, vocab, hidden = 40, 300, 128
+    xh = torch.randint(-2, 3, (rows, hidden), generator=gh).float().bfloat16()
+    wh = torch.randint(-2, 3, (vocab, hidden), generator=gh).float().bfloat16()
+    wh[250] = wh[17]
+    temps = np.array([0.5, 0.8, 1.0, 1.25, 2.0], dtype=np.float32)
+    logits = (xh.float() @ wh.float().T).bfloat16().to(torch.float64).numpy()
+    assert np.abs(logits).max() < 256
+    x0, p = oracle.confidence_argmax(logits.reshape(5, 8, vocab), temps)
+    save("lm_head.npz", x=bits(xh), w=bits(wh), temperatures=temps, rows_per_temp=np.int32(8),
+         x0=x0.reshape(-1).astype(np.int64), x0_p=p.reshape(-1).astype(np.float64))
 
 if __name__ == "__main__":
     main()

@@ -96,6 +96,26 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     assert sl(ctypes.c_void_p(18), 4096) == -3 and b"aligned" in L.mdx_last_error()
 
 
+def test_fused_head_and_calibration_arguments_are_validated(L):
+    null = None
+    one = ctypes.c_void_p(16)
+    ws = L.mdx_lm_head_confidence_workspace_bytes(1024, 151936)
+    assert ws == 1024 * 1188 * 16 and L.mdx_lm_head_confidence_workspace_bytes(0, 151936) == 0     # one record per row and 128-entry slice
+    big = ctypes.c_void_p(1 << 20)
+    head = lambda **kw: L.mdx_lm_head_confidence(                                                   # noqa: E731
+        kw.get("x", one), kw.get("xs", 2048), one, 2048, null, 1, null, one, one, kw.get("rows", 1024), 151936, kw.get("hidden", 2048),
+        kw.get("ws", big), kw.get("ws_bytes", ws), null)
+    assert head(x=null) == -1 and b"null" in L.mdx_last_error()
+    assert head(hidden=2000) == -2 and b"hidden" in L.mdx_last_error()
+    assert head(xs=2047) == -2
+    assert head(ws_bytes=ws - 16) == -3 and b"workspace" in L.mdx_last_error()
+    assert head(rows=0) == 0
+    assert L.mdx_calib_mfma_loop(7, one, one, 4, 8, null) == -1
+    assert L.mdx_calib_mfma_loop(32, null, one, 4, 8, null) == -1
+    assert L.mdx_calib_mfma_loop_flops(32, 256, 8) == 256 * 4 * 8 * 8 * 32 * 32 * 16 * 2
+    assert L.mdx_calib_mfma_loop_flops(16, 256, 3) == 256 * 4 * 8 * 16 * 16 * 16 * 32 * 2              # iterations rounded up to 8
+
+
 def test_ops_fail_loudly_off_gpu():
     import torch
     import mdx
@@ -116,7 +136,7 @@ def test_context_mirror():
 
 
 def test_generated_kernel_core_is_current():
-    """staircase_pair_core.inc and its fp16 twin are the committed outputs of their generator: regenerate and compare."""
+    """staircase_pair_core.inc, its fp16 twin and lm_head_core.inc are the committed outputs of their generators: regenerate and compare."""
     import subprocess
     import sys
     from pathlib import Path
@@ -125,3 +145,6 @@ def test_generated_kernel_core_is_current():
     assert out.stdout == (csrc / "staircase_pair_core.inc").read_text()
     out = subprocess.run([sys.executable, str(csrc / "gen_staircase_pair_core.py"), "f16"], capture_output=True, text=True, check=True)
     assert out.stdout == (csrc / "staircase_pair_core_f16.inc").read_text()
+    # the core of the fused vocabulary projection
+    out = subprocess.run([sys.executable, str(csrc / "gen_lm_head_core.py")], capture_output=True, text=True, check=True)
+    assert out.stdout == (csrc / "lm_head_core.inc").read_text()

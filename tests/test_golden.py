@@ -86,6 +86,20 @@ def test_oracle_reproduces_sampling_and_block_state_fixtures():
     assert b["phase"].tolist() == [1, 2, 1, 0, 2] and b["phase_after"].tolist() == [2, 0, 1, 0, 0]
 
 
+def test_oracle_reproduces_fused_head_fixture():
+    f = load("lm_head.npz")
+    x, w = bf16(f["x"]), bf16(f["w"])
+    logits = (x.float() @ w.float().T).bfloat16().to(torch.float64).numpy()
+    rpt = int(f["rows_per_temp"])
+    x0, p = oracle.confidence_argmax(logits.reshape(-1, rpt, logits.shape[1]), f["temperatures"])
+    assert np.array_equal(x0.reshape(-1), f["x0"]) and np.allclose(p.reshape(-1), f["x0_p"], rtol=1e-12)
+    # independent of the oracle: argmax / softmax by torch on the same exact logits, and the forced tie resolves to the lower index
+    t = torch.from_numpy(logits) / torch.from_numpy(f["temperatures"].astype(np.float32)).double().repeat_interleave(rpt)[:, None]
+    assert np.array_equal(torch.argmax(t, -1).numpy(), f["x0"])
+    np.testing.assert_allclose(torch.softmax(t, -1).max(-1).values.numpy(), f["x0_p"], rtol=1e-6)
+    assert 250 not in f["x0"].tolist()
+
+
 # ----------------------------------------------------------------------------- GPU: HIP path == fixtures
 @pytest.mark.gpu
 def test_hip_sampling_matches_fixtures(dev):
@@ -192,3 +206,13 @@ def test_hip_layer_ops_match_fixtures(dev):
         w = bf16(want).float()
         diff = (got.float().cpu() - w).abs()
         assert (diff <= w.abs() * 2 ** -7 + 1e-30).all() and (diff == 0).float().mean() > 0.97
+
+
+@pytest.mark.gpu
+def test_hip_fused_head_matches_fixture(dev):
+    import mdx
+    f = load("lm_head.npz")
+    x0, p = mdx.lm_head_confidence(bf16(f["x"]).to(dev), bf16(f["w"]).to(dev), torch.from_numpy(f["temperatures"]).to(dev),
+                                   rows_per_temp=int(f["rows_per_temp"]))
+    assert np.array_equal(x0.cpu().numpy(), f["x0"])
+    np.testing.assert_allclose(p.cpu().numpy(), f["x0_p"], rtol=3e-5)
