@@ -273,7 +273,10 @@ def epilogue_tile(xt):
             f"v_add_f32_e32 {SUM}, {s4[0]}, {s4[2]}",
             f"v_fma_f32 {T[0]}, {MS}, {C}, -{HM}",                          # m c - round(m c)
             f"v_exp_f32_e64 {T[0]}, -{T[0]}", "s_nop 1",
-            f"v_mul_f32_e32 {SUM}, {SUM}, {T[0]}"]
+            f"v_mul_f32_e32 {SUM}, {SUM}, {T[0]}",
+            # a lane all of whose logits lie beyond the vocabulary has m = -inf and a sum of 0 -- but the correction
+            # factor of the stand-in maximum is 2^(+-1e22), and 0 x inf is not 0: such a lane's sum is set to 0
+            f"v_cmp_lt_f32_e32 vcc, {NEG_INF}, {M}", f"v_cndmask_b32_e32 {SUM}, 0, {SUM}, vcc"]
     # merge the two half-wavefronts (lanes l and l + 32 hold the same x row): after the swaps both see both states
     M0_, M1_, S0_, S1_, G0_, G1_ = U[6], U[7], U[8], U[9], U[10], U[11]
     out += [f"v_mov_b32_e32 {M0_}, {M}", f"v_mov_b32_e32 {M1_}, {M}", f"v_mov_b32_e32 {S0_}, {SUM}", f"v_mov_b32_e32 {S1_}, {SUM}",

@@ -50,10 +50,10 @@ def test_prefill_random_shapes(dev):
 def test_paged_random_shapes(dev):
     import mdx
     rng = np.random.default_rng(4048)
-    for case in range(28):
+    for case in range(40):
         hq, hkv = HEADS[rng.integers(len(HEADS))]
         page = int(rng.choice([32, 64, 128, 256, 512, 96]))
-        sq = int(rng.choice([32, 32, 32, 1, 7, 16]))
+        sq = int(rng.choice([32, 32, 32, 1, 7, 16])) if case < 28 else int(rng.choice([33, 48, 64, 96, 100, 128]))    # blocks of up to 128 positions
         bs = int(rng.choice([1, 2, 3, 5, 8, 13, 24, 32, 40, 64, 70]))
         top = int(rng.choice([200, 700, 2500]))
         ctxs = [int(x) for x in rng.integers(0, top, bs)]
@@ -81,7 +81,7 @@ def test_paged_random_shapes(dev):
         print(f"paged case {case}: heads {hq}/{hkv} page {page} sq {sq} bs {bs} max ctx {max(ctxs)} width {bt.shape[1]}", flush=True)
         args = (q.to(dev), kc.to(dev), vc.to(dev))
         kw = dict(cache_seqlens=lens.to(dev), block_table=bt.to(dev), softmax_scale=scale, causal=False)
-        own = torch.zeros(4096, dtype=torch.float32, device=dev)
+        own = torch.zeros(8192, dtype=torch.float32, device=dev)
         one = mdx.flash_attn_with_kvcache(*args, **kw, counters=own)
         two = mdx.flash_attn_with_kvcache(*args, **kw, counters=False)
         torch.cuda.synchronize()
@@ -90,6 +90,77 @@ def test_paged_random_shapes(dev):
         assert err < TOL, f"case {case}: max-abs {err}"
         assert torch.equal(one, two), f"case {case}: one launch differs from two"
         assert own.abs().sum().item() == 0
+
+
+def test_prefill_random_shapes_with_many_sequences(dev):
+    """65 to 600 sequences per launch (the lookup of a workgroup's row group then walks them 64 at a time), lengths
+    from empty to a few row groups, occasionally one long sequence; both kernels (even and odd head ratios)."""
+    import mdx
+    rng = np.random.default_rng(909)
+    for case in range(10):
+        hq, hkv = HEADS[rng.integers(len(HEADS))]
+        S = int(rng.choice([4, 32, 32, 64, 128]))
+        B = int(rng.choice([65, 100, 128, 129, 257, 400, 600]))
+        top = int(rng.choice([40, 150, 500]))
+        lens = [int(x) for x in rng.integers(0, top, B)]
+        if case % 3 == 0:
+            lens[rng.integers(B)] = int(rng.integers(600, 1400))
+        g = torch.Generator().manual_seed(3000 + case)
+        N = sum(lens)
+        q = torch.randn(N, hq, 128, generator=g).bfloat16()
+        k = torch.randn(N, hkv, 128, generator=g).bfloat16()
+        v = torch.randn(N, hkv, 128, generator=g).bfloat16()
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        print(f"many-sequence case {case}: heads {hq}/{hkv} S {S} B {B} tokens {N} longest {max(lens)}", flush=True)
+        o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S, max_seqlen=max(lens))
+        torch.cuda.synchronize()
+        ref = oracle.staircase_attn_varlen(q, k, v, cu, S)
+        err = (o.float().cpu() - ref).abs().max().item()
+        assert err < TOL, f"case {case}: max-abs {err}"
+
+
+def test_fused_head_random_shapes(dev):
+    """Random row counts, vocabulary sizes (tile edges on both axes), hidden sizes, row strides, temperatures and
+    compacted rows: tokens equal to the oracle's on bf16(x @ W.T) up to near-ties of one bf16 step at the maximum."""
+    import mdx
+    rng = np.random.default_rng(31337)
+    for case in range(14):
+        rows = int(rng.choice([1, 5, 31, 64, 130, 255, 256, 257, 300, 513, 700]))
+        vocab = int(rng.choice([1, 100, 128, 129, 255, 256, 257, 1000, 4097, 20000]))
+        hidden = int(rng.choice([128, 256, 384, 1024, 2048]))
+        xs, ws = hidden + int(rng.choice([0, 8, 64])), hidden + int(rng.choice([0, 16]))
+        g = torch.Generator().manual_seed(7000 + case)
+        xbuf = torch.randn(rows, xs, generator=g).bfloat16()
+        wbuf = (torch.randn(vocab, ws, generator=g) * (3.0 / hidden ** 0.5)).bfloat16()
+        x, w = xbuf[:, :hidden], wbuf[:, :hidden]
+        n_temp = int(rng.choice([0, 1, 3]))
+        print(f"fused head case {case}: rows {rows} vocab {vocab} hidden {hidden} strides {xs}/{ws} temps {n_temp}", flush=True)
+        logits = (x.float() @ w.float().T).bfloat16().to(torch.float64).numpy()
+        if n_temp == 0:
+            x0, p = mdx.lm_head_confidence(xbuf.to(dev)[:, :hidden], wbuf.to(dev)[:, :hidden])
+            scaled = logits
+        else:
+            temps = torch.tensor(rng.uniform(0.5, 2.0, n_temp), dtype=torch.float32)
+            ids = torch.tensor(np.sort(rng.choice(n_temp * 16, size=rows, replace=rows > n_temp * 16)), dtype=torch.int64)
+            x0, p = mdx.lm_head_confidence(xbuf.to(dev)[:, :hidden], wbuf.to(dev)[:, :hidden], temps.to(dev), rows_per_temp=16, row_ids=ids.to(dev))
+            scaled = (logits.astype(np.float32) / temps.numpy()[ids.numpy() // 16][:, None]).astype(np.float64)
+        torch.cuda.synchronize()
+        ex0 = scaled.argmax(-1)
+        e = np.exp(scaled - scaled.max(-1, keepdims=True))
+        ep = e[np.arange(rows), ex0] / e.sum(-1)
+        got = x0.cpu().numpy()
+        top = logits[np.arange(rows), logits.argmax(-1)]
+        step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(top), 2.0 ** -100))) - 7)
+        same = got == ex0
+        assert np.all(same | (logits[np.arange(rows), got] >= top - step)), f"case {case}: a pick that is not a near-tie of the maximum"
+        if rows >= 64:
+            assert same.mean() > 0.95
+        # a logit one bf16 step off (another order of summation, a sum on a rounding boundary) moves a probability by up to
+        # exp(step / T) - 1 of itself: the tolerance of a row follows from its own largest logit and temperature
+        T_row = np.ones(rows) if n_temp == 0 else temps.numpy()[ids.numpy() // 16].astype(np.float64)
+        tol = np.expm1(step / T_row) * 1.1 + 1e-4
+        rel = np.abs(p.cpu().numpy() - ep) / ep
+        assert np.all(rel[same] <= tol[same]), f"case {case}: confidence off by {rel[same].max()} (allowed {tol[same][rel[same].argmax()]})"
 
 
 def test_filter_and_seeded_sampling_random_shapes(dev):
