@@ -43,7 +43,7 @@ extern "C" {
 
 #define MDX_BF16 0                 /* q/k/v/o, the caches, the layer ops, the logits */
 #define MDX_F16  1                 /* q/k/v/o and the caches of the two attention calls, the logits */
-#define MDX_F32  2                 /* logits only */
+#define MDX_F32  2                 /* the logits; q/k/v/o and the caches of the two attention calls (fp32 arithmetic) */
 
 typedef void* mdx_stream_t;        /* hipStream_t */
 
@@ -91,12 +91,17 @@ int mdx_store_kvcache(const void* key, const void* value,
  * sizes the grid, and rows of a longer sequence beyond it are never computed
  * (their o rows keep what they held; the lengths are on the device, so the
  * call cannot check this).  total_tokens is always a valid bound; the
- * reference interface has no such argument.  Supported: d a multiple of 16
- * up to 128 (the reference kernel takes BLOCK_DMODEL = head_dim, :183; widths
- * below 128 run as 128 with zero padding, in the one-head-per-wavefront
- * kernel, and only d columns of o are written), dtype MDX_BF16 or MDX_F16
- * (the reference kernel takes q's dtype, :179-197; both run the same
- * kernels, fp16 within a few percent of bf16).
+ * reference interface has no such argument.  Supported: the reference kernel
+ * takes q's dtype (:179-197) and BLOCK_DMODEL = head_dim (:183).  MDX_BF16 and
+ * MDX_F16 with d a multiple of 16 up to 128 run on the 16-bit matrix
+ * instructions (both the same kernels, fp16 within a few percent of bf16;
+ * widths below 128 run as 128 with zero padding, in the one-head-per-wavefront
+ * kernel, and only d columns of o are written; tensors 16-byte aligned with
+ * strides that are multiples of 8 elements, o's of 4).  MDX_F32, and 16-bit
+ * tensors whose d is another multiple of 4 up to 256, run in fp32 arithmetic
+ * on the fp32 matrix instruction (probabilities never rounded, 16-bit inputs
+ * widened; exact rather than fast: about a fifteenth of the 16-bit kernels' rate;
+ * tensors aligned to four elements with strides that are multiples of 4).
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                               int64_t q_stride_t, int64_t q_stride_h,
@@ -129,10 +134,13 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * kernel picks it from the lengths); its size comes from
  * mdx_paged_block_attn_workspace_bytes with the same shape arguments, and its
  * contents need no initialisation.
- * Supported: d a multiple of 16 up to 128 (narrower heads are padded with zeros on the way into LDS; the
- * partials keep their 128-wide layout), Sq <= 128 (blocks longer than 32 positions run as tiles of 32 queries
- * that stream the same keys; any Hq that is a multiple of Hkv), page_size % 32 == 0,
- * MDX_BF16 or MDX_F16.
+ * Supported: Sq <= 128 (blocks longer than 32 positions run as tiles of 32 queries that stream the same keys), any Hq
+ * that is a multiple of Hkv, page_size % 32 == 0.  MDX_BF16 and MDX_F16 with d a multiple of 16 up to 128 run on the
+ * 16-bit matrix instructions (narrower heads are padded with zeros on the way into LDS; the partials keep their
+ * 128-wide layout).  MDX_F32, and 16-bit tensors whose d is another multiple of 4 up to 256 (flash-attn takes heads
+ * of up to 256 columns), run in fp32 arithmetic on the fp32 matrix instruction: one workgroup per (sequence, KV head,
+ * query tile) walks the whole context, no split and no workspace (the workspace query returns 0 for those widths; a
+ * workspace that is passed anyway is ignored); exact rather than fast.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,
                                              int32_t num_kv_heads, int32_t head_dim,

@@ -17,7 +17,7 @@ CSRC = ROOT / "csrc"
 OBJ = ROOT / "build"
 LIB = ROOT / "mdx" / "libmdx.so"
 
-SOURCES = ["mdx_api.hip", "store_kvcache.hip", "unmask.hip", "logit_filter.hip", "staircase_attn.hip", "paged_attn.hip", "paged_attn_static.hip", "qk_norm_rope_store.hip", "layer_ops.hip", "block_state.hip", "lm_head_unmask.hip", "calib_probe.hip"]
+SOURCES = ["mdx_api.hip", "store_kvcache.hip", "unmask.hip", "logit_filter.hip", "staircase_attn.hip", "staircase_attn_f32.hip", "paged_attn.hip", "paged_attn_f32.hip", "paged_attn_static.hip", "qk_norm_rope_store.hip", "layer_ops.hip", "block_state.hip", "lm_head_unmask.hip", "calib_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -596,6 +596,7 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
                                                         int32_t max_pages, int32_t page_size)
 {
     if (bs <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pages <= 0 || page_size <= 0) return 0;
+    if (head_dim > kHeadDim || head_dim % 16 != 0) return 0;       // the fp32-arithmetic kernel: no split, no partials
     const int G = num_q_heads / num_kv_heads;
     const int HPW = (G % 2 == 0) ? 2 : 1;
     const int nqt = sq <= kQTile ? 1 : (sq + kQTile - 1) / kQTile;
@@ -607,6 +608,15 @@ extern "C" int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, 
 }
 
 namespace mdx {
+
+int launch_paged_f32(const void* q, void* o, const void* k_cache, const void* v_cache,
+                     int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                     int64_t o_stride_b, int64_t o_stride_s, int64_t o_stride_h,
+                     int64_t cache_stride_page, int64_t cache_stride_tok, int64_t cache_stride_head,
+                     const int32_t* block_table, int64_t bt_stride, const int32_t* context_lens,
+                     int32_t bs, int32_t sq, int32_t num_q_heads, int32_t num_kv_heads,
+                     int32_t head_dim, int32_t max_pages, int32_t page_size, int64_t num_pages,
+                     float scale, int32_t dtype, hipStream_t stream);                         // paged_attn_f32.hip
 
 // The launch behind every paged entry point of the library.
 int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cache,
@@ -622,9 +632,12 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(bs >= 0 && sq >= 0 && max_pages >= 0 && num_pages >= 0, MDX_EINVAL, "paged_block_attn: negative size");
-    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "paged_block_attn: dtype %d (bf16 or fp16)", dtype);
-    MDX_REQUIRE(head_dim >= 16 && head_dim <= kHeadDim && head_dim % 16 == 0, MDX_EUNSUPPORTED,
-                "paged_block_attn: head_dim %d (multiples of 16 up to 128)", head_dim);
+    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16 || dtype == MDX_F32, MDX_EUNSUPPORTED, "paged_block_attn: dtype %d (bf16, fp16 or fp32)", dtype);
+    // 16-bit elements and heads of 16, 32, ..., 128 columns run on the 16-bit matrix instructions; fp32 tensors and
+    // the other head widths up to 256 on the fp32 one (paged_attn_f32.hip: no split, no workspace)
+    const bool f32_arithmetic = dtype == MDX_F32 || head_dim > kHeadDim || head_dim % 16 != 0;
+    MDX_REQUIRE(head_dim >= 4 && head_dim <= 256 && head_dim % 4 == 0, MDX_EUNSUPPORTED,
+                "paged_block_attn: head_dim %d (multiples of 4 up to 256)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "paged_block_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
     MDX_REQUIRE(sq <= kMaxSq, MDX_EUNSUPPORTED, "paged_block_attn: %d queries per sequence (max %d)", sq, kMaxSq);
@@ -635,6 +648,10 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     MDX_REQUIRE(max_pages > 0, MDX_EINVAL, "paged_block_attn: empty block table");
     MDX_REQUIRE(q && o && k_cache && v_cache && block_table && context_lens, MDX_EINVAL, "paged_block_attn: null pointer");
     MDX_REQUIRE(bt_stride >= max_pages, MDX_EINVAL, "paged_block_attn: bt_stride < max_pages");
+    if (f32_arithmetic)
+        return launch_paged_f32(q, o, k_cache, v_cache, q_stride_b, q_stride_s, q_stride_h, o_stride_b, o_stride_s, o_stride_h,
+                                cache_stride_page, cache_stride_tok, cache_stride_head, block_table, bt_stride, context_lens,
+                                bs, sq, num_q_heads, num_kv_heads, head_dim, max_pages, page_size, num_pages, scale, dtype, stream);
     MDX_REQUIRE(mdx::aligned16(q) && mdx::aligned16(o) && mdx::aligned16(k_cache) && mdx::aligned16(v_cache) &&
                 q_stride_b % 8 == 0 && q_stride_s % 8 == 0 && q_stride_h % 8 == 0 &&
                 o_stride_b % 8 == 0 && o_stride_s % 8 == 0 && o_stride_h % 8 == 0 &&

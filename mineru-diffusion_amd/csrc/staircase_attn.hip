@@ -425,6 +425,15 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_pair_kernel(const Stair
 
 }  // namespace
 
+namespace mdx {
+int launch_staircase_f32(const void* q, const void* k, const void* v, void* o,
+                         int64_t q_stride_t, int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h,
+                         int64_t v_stride_t, int64_t v_stride_h, int64_t o_stride_t, int64_t o_stride_h,
+                         const int32_t* cu_seqlens, int32_t batch, int64_t max_l,
+                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                         int32_t log2_s, float scale, int32_t dtype, hipStream_t stream);      // staircase_attn_f32.hip
+}
+
 extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
                                          int64_t q_stride_t, int64_t q_stride_h,
                                          int64_t k_stride_t, int64_t k_stride_h,
@@ -438,9 +447,12 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     MDX_REQUIRE(batch >= 0 && total_tokens >= 0 && max_seqlen >= 0, MDX_EINVAL, "staircase_attn: negative size");
-    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (bf16 or fp16)", dtype);
-    MDX_REQUIRE(head_dim >= 16 && head_dim <= kHeadDim && head_dim % 16 == 0, MDX_EUNSUPPORTED,
-                "staircase_attn: head_dim %d (multiples of 16 up to 128)", head_dim);
+    MDX_REQUIRE(dtype == MDX_BF16 || dtype == MDX_F16 || dtype == MDX_F32, MDX_EUNSUPPORTED, "staircase_attn: dtype %d (bf16, fp16 or fp32)", dtype);
+    // 16-bit elements and heads of 16, 32, ..., 128 columns run on the 16-bit matrix instructions; everything else that
+    // the reference's kernel takes (fp32 tensors, heads of up to 256 columns) on the fp32 one (staircase_attn_f32.hip)
+    const bool f32_arithmetic = dtype == MDX_F32 || head_dim > kHeadDim || head_dim % 16 != 0;
+    MDX_REQUIRE(head_dim >= 4 && head_dim <= 256 && head_dim % 4 == 0, MDX_EUNSUPPORTED,
+                "staircase_attn: head_dim %d (multiples of 4 up to 256)", head_dim);
     MDX_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, MDX_EINVAL,
                 "staircase_attn: Hq %d not a multiple of Hkv %d", num_q_heads, num_kv_heads);
     int log2_s = -1;
@@ -450,6 +462,12 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     if (batch == 0 || total_tokens == 0 || max_seqlen == 0) return MDX_OK;
     MDX_REQUIRE(q && k && v && o && cu_seqlens_q && cu_seqlens_k, MDX_EINVAL, "staircase_attn: null pointer");
     MDX_REQUIRE(total_tokens < ((int64_t)1 << 31) - 256, MDX_EUNSUPPORTED, "staircase_attn: too many tokens");
+    if (f32_arithmetic) {
+        const int64_t longest = max_seqlen < total_tokens ? max_seqlen : total_tokens;
+        return mdx::launch_staircase_f32(q, k, v, o, q_stride_t, q_stride_h, k_stride_t, k_stride_h, v_stride_t, v_stride_h,
+                                         o_stride_t, o_stride_h, cu_seqlens_k, batch, longest, num_q_heads, num_kv_heads, head_dim,
+                                         log2_s, scale, dtype, stream);
+    }
     // 16-byte vector access to every row of q/k/v, 8-byte to o
     MDX_REQUIRE(mdx::aligned16(q) && mdx::aligned16(k) && mdx::aligned16(v) && mdx::aligned16(o) &&
                 q_stride_t % 8 == 0 && q_stride_h % 8 == 0 && k_stride_t % 8 == 0 && k_stride_h % 8 == 0 &&

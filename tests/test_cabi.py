@@ -60,19 +60,20 @@ def test_bad_arguments_are_refused_without_a_launch(L):
     sa = lambda **kw: L.mdx_staircase_attn_varlen(                                            # noqa: E731
         one, one, one, one, 2048, 128, 1024, 128, 1024, 128, 2048, 128, one, one, 1, 100, 100,
         kw.get("hq", 16), kw.get("hkv", 8), kw.get("d", 128), kw.get("S", 32), kw.get("scale", 0.1), kw.get("dtype", 0), null)
-    assert sa(d=256) == -2 and b"head_dim" in L.mdx_last_error()
-    assert sa(d=72) == -2 and b"head_dim" in L.mdx_last_error()     # narrow heads: multiples of 16 only
+    assert sa(d=260) == -2 and b"head_dim" in L.mdx_last_error()    # up to 256 columns (above 128: the fp32-arithmetic kernel)
+    assert sa(d=70) == -2 and b"head_dim" in L.mdx_last_error()     # multiples of 4 only
     assert sa(S=48) == -1 and b"staircase_size" in L.mdx_last_error()
     assert sa(hq=12) == -1
-    assert sa(dtype=2) == -2                                   # fp32 q/k/v: the attention runs on 16-bit elements only
+    assert sa(dtype=3) == -2 and b"dtype" in L.mdx_last_error()     # bf16, fp16 and fp32 are the element types
     assert sa(scale=-1.0) == -1
     pa = lambda **kw: L.mdx_paged_block_attn(                                                  # noqa: E731
         one, one, one, one, 65536, 2048, 128, 65536, 2048, 128, 262144, 1024, 128, one, 17, one,
         4, kw.get("sq", 32), 16, 8, kw.get("d", 128), 17, kw.get("page", 256), 100, 0.1, 0, kw.get("ws", null), kw.get("ws_bytes", 0), null)
     assert pa(sq=129) == -2 and b"queries per sequence" in L.mdx_last_error()    # up to four tiles of 32 queries
     assert pa(page=100) == -2
-    assert pa(d=256) == -2 and b"head_dim" in L.mdx_last_error()
-    assert pa(d=40) == -2
+    assert pa(d=260) == -2 and b"head_dim" in L.mdx_last_error()    # up to 256 columns (above 128: the fp32-arithmetic kernel)
+    assert pa(d=42) == -2                                           # multiples of 4 only
+    assert L.mdx_paged_block_attn_workspace_bytes(16, 32, 16, 8, 256, 17, 256) == 0     # that kernel never splits a sequence
     assert pa() == -3 and b"workspace" in L.mdx_last_error()
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, -1, one, one, 2, 32, null) == -1      # k < 0
     assert L.mdx_select_transfer(one, one, one, 7, 0.9, 1, one, one, 2, 2000, null) == -2      # block too long
