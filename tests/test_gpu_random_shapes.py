@@ -211,3 +211,59 @@ def test_filter_and_seeded_sampling_random_shapes(dev):
         kept_mask = torch.isfinite(f.float()).view(bs, S, V)
         assert bool(kept_mask.gather(-1, a[0].unsqueeze(-1)).all())      # a drawn token is always one that survived the filter
     assert checked > 100
+
+
+def test_fp32_arithmetic_attention_random_shapes(dev):
+    """Both attention calls on element types and head widths that run in fp32 arithmetic (fp32 tensors; 16-bit tensors
+    whose head is wider than 128 columns or not a multiple of 16): random batches, lengths, head layouts, staircase,
+    block and page sizes.  fp32 tensors within 3e-5 of the fp32 oracle, 16-bit ones within their output rounding."""
+    import mdx
+    rng = np.random.default_rng(777)
+    widths16 = [8, 24, 40, 72, 100, 136, 160, 200, 256]
+    for case in range(30):
+        if case % 3 == 0:
+            dtype, d = torch.float32, int(rng.choice([4, 32, 64, 96, 128, 192, 256]))
+        else:
+            dtype, d = (torch.bfloat16 if case % 3 == 1 else torch.float16), int(rng.choice(widths16))
+        tol = 3e-5 if dtype == torch.float32 else 1e-2
+        hq, hkv = HEADS[rng.integers(len(HEADS))]
+        g = torch.Generator().manual_seed(5000 + case)
+        # prefill
+        S = int(2 ** rng.integers(0, 8))
+        B = int(rng.integers(1, 5))
+        lens = [int(x) for x in rng.integers(0, 300, B)]
+        if sum(lens) == 0:
+            lens[0] = 7
+        N = sum(lens)
+        q = torch.randn(N, hq, d, generator=g).to(dtype)
+        k = torch.randn(N, hkv, d, generator=g).to(dtype)
+        v = torch.randn(N, hkv, d, generator=g).to(dtype)
+        cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32)
+        print(f"case {case}: {dtype} d {d} heads {hq}/{hkv} S {S} lens {lens}", flush=True)
+        o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), S)
+        torch.cuda.synchronize()
+        err = (o.float().cpu() - oracle.staircase_attn_varlen(q, k, v, cu, S)).abs().max().item()
+        assert err < tol, f"prefill case {case}: max-abs {err}"
+        # paged
+        page = int(rng.choice([32, 64, 256]))
+        sq = int(rng.integers(1, 70))
+        ctxs = [int(x) for x in rng.integers(0, 700, int(rng.integers(1, 5)))]
+        maxp = max(1, max((c + page - 1) // page for c in ctxs))
+        pool = sum((c + page - 1) // page for c in ctxs) + 3
+        qp = torch.randn(len(ctxs), sq, hq, d, generator=g).to(dtype)
+        kc = torch.randn(pool, page, hkv, d, generator=g).to(dtype)
+        vc = torch.randn(pool, page, hkv, d, generator=g).to(dtype)
+        perm = torch.randperm(pool, generator=g)
+        bt = torch.full((len(ctxs), maxp), -1, dtype=torch.int32)
+        at = 0
+        for b, c in enumerate(ctxs):
+            n = (c + page - 1) // page
+            bt[b, :n] = perm[at:at + n].to(torch.int32)
+            at += n
+        lens_d = torch.tensor(ctxs, dtype=torch.int32)
+        print(f"case {case}: paged sq {sq} page {page} ctxs {ctxs}", flush=True)
+        od = mdx.flash_attn_with_kvcache(qp.to(dev), kc.to(dev), vc.to(dev), cache_seqlens=lens_d.to(dev), block_table=bt.to(dev),
+                                         softmax_scale=1 / math.sqrt(d), causal=False)
+        torch.cuda.synchronize()
+        err = (od.float().cpu() - oracle.paged_block_attn(qp, kc, vc, bt, lens_d, 1 / math.sqrt(d))).abs().max().item()
+        assert err < tol, f"paged case {case}: max-abs {err}"
