@@ -457,7 +457,7 @@ def main():
     ap.add_argument("--skip-cpu", action="store_true", help="leave out the CPU baseline leg (profiling runs)")
     ap.add_argument("--no-full-logits-leg", action="store_true",
                     help="decode leg: skip the second generation that projects all 32 positions of every block")
-    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,lmhead,decode (default all; gumbel and filter run inside unmask), plus power (only when named: socket power and clock under the attention kernel and the library GEMM)")
+    ap.add_argument("--only", default="", help="comma list of legs to run: calib,step,store,paged,unmask,gumbel,filter,lmhead,decode (default all; gumbel and filter run inside unmask), plus power (only when named: socket power and clock under the attention kernel and the library GEMM) and f32 (only when named: the attention calls on fp32 tensors)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); run with --gpus 1")
@@ -610,6 +610,38 @@ def main():
                 time.sleep(0.5)
             del zf, z, a_r, a_z, p_ops, p_out, hw, hx, hws
             torch.cuda.empty_cache()
+    if "f32" in only:
+        # The two attention calls in fp32 arithmetic (fp32 tensors; the path of head widths outside the 16-bit kernels):
+        # a compatibility path, timed only when named.  Prefill: four sequences of 2048 tokens and one of 8192, fp32,
+        # d = 128; paged: 16 sequences of 2700 keys.  Roofline: the fp32 matrix instruction's published peak.
+        f32 = {}
+        for name, lens in (("prefill_4x2048", [2048] * 4), ("prefill_1x8192", [8192])):
+            n_tok = sum(lens)
+            qf = torch.randn(n_tok, HQ, D, device=dev)
+            kf = torch.randn(n_tok, HKV, D, device=dev)
+            vf = torch.randn(n_tok, HKV, D, device=dev)
+            cu = torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=dev)
+            ms, _ = time_kernel(lambda i: mdx.sparse_attn_varlen(qf, kf, vf, cu, cu, S, max_seqlen=max(lens)), 2, 5, graph=True)
+            flops = cfg3_work(lens)["flops"]
+            f32[name] = dict(ms=round(ms, 4), roofline=dict(bound="mfma", achieved=round(flops / ms / 1e9, 1), peak=157.3, unit="TFLOP/s",
+                                                            frac=round(flops / ms / 1e9 / 157.3, 4), traffic=None))
+            del qf, kf, vf
+        bs_p, ctx_p = 16, 2700
+        pages_p = (ctx_p + PAGE - 1) // PAGE
+        qp = torch.randn(bs_p, S, HQ, D, device=dev)
+        kcp = torch.randn(bs_p * pages_p, PAGE, HKV, D, device=dev)
+        vcp = torch.randn(bs_p * pages_p, PAGE, HKV, D, device=dev)
+        btp = torch.arange(bs_p * pages_p, dtype=torch.int32, device=dev).view(bs_p, pages_p)
+        lens_p = torch.full((bs_p,), ctx_p, dtype=torch.int32, device=dev)
+        ms, _ = time_kernel(lambda i: mdx.flash_attn_with_kvcache(qp, kcp, vcp, cache_seqlens=lens_p, block_table=btp, softmax_scale=D ** -0.5,
+                                                                  causal=False), 2, 5, graph=True)
+        flops = 4.0 * S * HQ * D * bs_p * ctx_p
+        f32["paged_16x2700"] = dict(ms=round(ms, 4), roofline=dict(bound="mfma", achieved=round(flops / ms / 1e9, 1), peak=157.3, unit="TFLOP/s",
+                                                                    frac=round(flops / ms / 1e9 / 157.3, 4), traffic=None))
+        result_ops["attention_fp32_arithmetic"] = f32
+        log(f"[bench] fp32-arithmetic attention: {f32}")
+        del qp, kcp, vcp
+        torch.cuda.empty_cache()
     if want("store"):
         # three rotating (source, cache) sets, about 900 MB touched per round trip, so the 256 MB
         # last-level cache cannot serve the next launch; the C ABI is called directly
