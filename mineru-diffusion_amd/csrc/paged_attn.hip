@@ -2,10 +2,10 @@
 // denoising block of every sequence attend, non-causally, to the first
 // context_lens[b] keys of that sequence's paged KV cache.  A workgroup serves one
 // tile of 32 queries; blocks of 64 or 128 positions (the reference's block length
-// is a configuration field, nanovllm/config.py:48) run as 2 or 4 query tiles on
-// the grid's z axis, each with its own partials and arrival counter, and stream
-// the same keys (which the tiles of a pair, launched next to each other, mostly
-// find in the L2 that the first of them filled).
+// is a configuration field, nanovllm/config.py:48) run as 2 or 4 query tiles,
+// each a workgroup with its own partials and arrival counter; they stream the
+// same keys and are launched next to each other, 8 workgroups apart, so that
+// they run on one XCD and the later ones find in its L2 what the first fetched.
 //
 // Replaces flash_attn_with_kvcache(..., causal=False) at
 // engines/nano_dvlm/nanovllm/layers/sdar_attention.py:48-56.
@@ -217,8 +217,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
-    const int hg = blockIdx.x;
-    const int qt = blockIdx.z;                      // this workgroup's tile of 32 queries
+    // launch order: head group fastest, then the query tiles of a (sequence, split), then the pairs -- the tiles of a
+    // block longer than 32 queries stream the same keys, so they start next to each other and on the same XCD
+    const int n_groups = P.num_q_heads / HPW;
+    const int hg = blockIdx.x % n_groups;
+    const int qt = blockIdx.x / n_groups;           // this workgroup's tile of 32 queries
     const int kw = wave % KW;                       // this wavefront's key slice
     const int head = hg * HPW + wave / KW;          // and query head
 
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             // (Quotients by reciprocal: an estimate is all that is needed, and every workgroup makes the same one;
             // the "+ 1" keeps the longest sequence within nsplit pieces whatever the rounding.)
             const int total = wave_sum(ctx_l), longest = wave_max(ctx_l), live = wave_sum(ctx_l > 0 ? 1 : 0);
-            const float per_group = (float)P.fit_slots * __builtin_amdgcn_rcpf((float)(gridDim.x * gridDim.z));      // resident workgroups per head group and query tile
+            const float per_group = (float)P.fit_slots * __builtin_amdgcn_rcpf((float)gridDim.x);      // resident workgroups per head group and query tile
             const float room = fmaxf(1.f, per_group - 0.5f * (float)live);
             const float least = (float)total * (1.f / 256.f) + (float)live <= 0.5f * per_group ? 256.f : 512.f;
             const float depth = __builtin_amdgcn_sqrtf(27.6f * (float)longest);
@@ -256,11 +259,11 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
             n = splits_of_lane();
             // a tile more per step (24 steps double the smallest split); a few workgroups beyond what is resident
             // may stay: the last to start are remainders, which fill the tail
-            for (int it = 0; it < 24 && wave_sum(n) * (int)(gridDim.x * gridDim.z) > P.fit_slots + P.fit_slots / 32; ++it) {
+            for (int it = 0; it < 24 && wave_sum(n) * (int)gridDim.x > P.fit_slots + P.fit_slots / 32; ++it) {
                 span += 64;
                 n = splits_of_lane();
             }
-            if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) *P.span_out = (float)span;
+            if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
         } else {
             if (P.span_out) {
                 // With a (sequence, head group) pair per CU the sequences are best left whole (no partials,
@@ -271,7 +274,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
                 const int live = wave_sum(ctx_l > 0 ? 1 : 0);
                 const int mean = wave_sum(ctx_l) / max(live, 1);
                 span = max(span, (mean + mean / 4 + kChunkAlign - 1) / kChunkAlign * kChunkAlign);
-                if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid == 0) *P.span_out = (float)span;
+                if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) *P.span_out = (float)span;
             }
             n = splits_of_lane();
         }
@@ -509,7 +512,7 @@ __global__ __launch_bounds__(64 * WAVES, (WAVES / HPW == 2) ? 2 : 1) void paged_
     __shared__ int i_am_last;
     wait_vector_memory();
     __syncthreads();
-    float* counter = P.arrive + ((int64_t)b * gridDim.x + hg) * P.nqt + qt;
+    float* counter = P.arrive + ((int64_t)b * n_groups + hg) * P.nqt + qt;
     if (tid == 0) i_am_last = atomicAdd(counter, 1.0f) == (float)(n_valid_splits - 1) ? 1 : 0;
     __syncthreads();
     if (!i_am_last) return;
@@ -710,7 +713,7 @@ int launch_paged(const void* q, void* o, const void* k_cache, const void* v_cach
     // With device-chosen splits of at least 1.25 x the mean length, sum_b ceil(len_b / split) <= 1.8 bs:
     // the dense numbering never needs more than 2 bs (sequence, split) pairs, whatever nsplit allows.
     const int pairs_y = device_span ? (bs * P.nsplit < 2 * bs ? bs * P.nsplit : 2 * bs) : bs * P.nsplit;
-    const dim3 grid((unsigned)(num_q_heads / HPW), (unsigned)pairs_y, (unsigned)P.nqt);
+    const dim3 grid((unsigned)(num_q_heads / HPW * P.nqt), (unsigned)pairs_y);
     // Up to one (sequence, head group) pair per CU: workgroups of 8 wavefronts on 128-key tiles, so that a
     // CU that holds a single workgroup still has two wavefronts per SIMD (batch 32 x 8 KV heads: 79 -> 69 us
     // on equal lengths); with more pairs than CUs the second round costs more than that gains.
