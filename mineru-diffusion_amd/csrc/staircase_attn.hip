@@ -429,7 +429,7 @@ namespace mdx {
 int launch_staircase_f32(const void* q, const void* k, const void* v, void* o,
                          int64_t q_stride_t, int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h,
                          int64_t v_stride_t, int64_t v_stride_h, int64_t o_stride_t, int64_t o_stride_h,
-                         const int32_t* cu_seqlens, int32_t batch, int64_t max_l,
+                         const int32_t* cu_seqlens, int32_t batch, int64_t max_l, int64_t total_tokens,
                          int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                          int32_t log2_s, float scale, int32_t dtype, hipStream_t stream);      // staircase_attn_f32.hip
 }
@@ -465,7 +465,7 @@ extern "C" int mdx_staircase_attn_varlen(const void* q, const void* k, const voi
     if (f32_arithmetic) {
         const int64_t longest = max_seqlen < total_tokens ? max_seqlen : total_tokens;
         return mdx::launch_staircase_f32(q, k, v, o, q_stride_t, q_stride_h, k_stride_t, k_stride_h, v_stride_t, v_stride_h,
-                                         o_stride_t, o_stride_h, cu_seqlens_k, batch, longest, num_q_heads, num_kv_heads, head_dim,
+                                         o_stride_t, o_stride_h, cu_seqlens_k, batch, longest, total_tokens, num_q_heads, num_kv_heads, head_dim,
                                          log2_s, scale, dtype, stream);
     }
     // 16-byte vector access to every row of q/k/v, 8-byte to o

@@ -24,7 +24,7 @@ struct WideParams {
     const void* q; const void* k; const void* v; void* o;
     int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh;    // strides in elements
     const int32_t* cu_seqlens;
-    int batch, n_row_groups, num_q_heads, num_kv_heads, head_dim, log2_s;
+    int batch, total_tokens, n_row_groups, num_q_heads, num_kv_heads, head_dim, log2_s;
     float c;                                                   // scale * log2(e)
 };
 
@@ -40,8 +40,10 @@ __global__ __launch_bounds__(kThreads, 1) void staircase_attn_f32_kernel(const W
     const int rg = P.n_row_groups - 1 - (int)blockIdx.y;       // the heaviest row groups start first
     const int b = blockIdx.z;
 
-    const int seq0 = P.cu_seqlens[b];
-    const int L = P.cu_seqlens[b + 1] - seq0;
+    // bounds that do not describe a range inside the packed tensors (decreasing, negative, past total_tokens) are clipped
+    // to one, so that no row outside q/k/v/o is ever touched
+    const int seq0 = min(max(P.cu_seqlens[b], 0), P.total_tokens);
+    const int L = min(max(P.cu_seqlens[b + 1], seq0), P.total_tokens) - seq0;
     if (L <= 0) return;
     const int S = 1 << P.log2_s;
     const int Lp = ((L + S - 1) >> P.log2_s) << P.log2_s;      // padded length
@@ -118,7 +120,7 @@ namespace mdx {
 int launch_staircase_f32(const void* q, const void* k, const void* v, void* o,
                          int64_t q_stride_t, int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h,
                          int64_t v_stride_t, int64_t v_stride_h, int64_t o_stride_t, int64_t o_stride_h,
-                         const int32_t* cu_seqlens, int32_t batch, int64_t max_l,
+                         const int32_t* cu_seqlens, int32_t batch, int64_t max_l, int64_t total_tokens,
                          int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                          int32_t log2_s, float scale, int32_t dtype, hipStream_t stream)
 {
@@ -135,6 +137,7 @@ int launch_staircase_f32(const void* q, const void* k, const void* v, void* o,
     P.v_st = v_stride_t; P.v_sh = v_stride_h; P.o_st = o_stride_t; P.o_sh = o_stride_h;
     P.cu_seqlens = cu_seqlens;
     P.batch = batch;
+    P.total_tokens = (int)total_tokens;
     P.n_row_groups = (int)((max_l + (1 << log2_s) - 1 + kRowsPerWg - 1) / kRowsPerWg);
     P.num_q_heads = num_q_heads; P.num_kv_heads = num_kv_heads; P.head_dim = head_dim; P.log2_s = log2_s;
     P.c = scale * kLog2e;

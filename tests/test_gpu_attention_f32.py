@@ -240,3 +240,19 @@ def test_decode_matches_prefill_last_block_in_fp32(dev):
     o2 = mdx.flash_attn_with_kvcache(q[-8:][None].to(dev), kc.to(dev), vc.to(dev), cache_seqlens=torch.tensor([L], dtype=torch.int32, device=dev),
                                      block_table=table.to(dev), softmax_scale=1 / math.sqrt(d), causal=False)
     assert (o1[-8:] - o2[0]).abs().max().item() < TOL_F32
+
+
+def test_fp32_sequence_bounds_are_clipped_to_the_tensors(dev):
+    """cu_seqlens that run past the packed tensors (or backwards) are clipped to them: no row outside q/k/v/o is touched."""
+    import mdx
+    g = torch.Generator().manual_seed(81)
+    q, k, v, cu = _packed(g, [200], 4, 2, 64, torch.float32)
+    good = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), cu.to(dev), cu.to(dev), 32)
+    long = torch.tensor([0, 250], dtype=torch.int32)
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), long.to(dev), long.to(dev), 32)
+    assert torch.equal(o, good)
+    back = torch.tensor([0, 120, 60, 200], dtype=torch.int32)           # the second sequence runs backwards: empty
+    o = mdx.sparse_attn_varlen(q.to(dev), k.to(dev), v.to(dev), back.to(dev), back.to(dev), 32)
+    torch.cuda.synchronize()
+    ref = oracle.staircase_attn_varlen(q[:120], k[:120], v[:120], torch.tensor([0, 120], dtype=torch.int32), 32)
+    assert (o[:60].cpu() - ref[:60]).abs().max().item() < TOL_F32
