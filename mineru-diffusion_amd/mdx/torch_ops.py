@@ -15,6 +15,7 @@ say what it returns without running: that is what this module adds.  Importing i
     torch.ops.mdx.rms_norm(x, weight, eps) -> y
     torch.ops.mdx.add_rms_norm(x, residual, weight, eps) -> (y, new_residual)
     torch.ops.mdx.silu_and_mul(x) -> y
+    torch.ops.mdx.lm_head_confidence(x, weight, temperatures) -> (x0, x0_p)
 
 Same kernels, same results as the functions of `mdx.ops` they wrap; nothing here computes.
 """
@@ -113,3 +114,14 @@ def silu_and_mul(x: Tensor) -> Tensor:
 @silu_and_mul.register_fake
 def _(x):
     return x.new_empty((*x.shape[:-1], x.shape[-1] // 2))
+
+
+@custom_op("mdx::lm_head_confidence", mutates_args=())
+def lm_head_confidence(x: Tensor, weight: Tensor, temperatures: Tensor | None) -> tuple[Tensor, Tensor]:
+    return ops.lm_head_confidence(x, weight, temperatures)
+
+
+@lm_head_confidence.register_fake
+def _(x, weight, temperatures):
+    lead = x.shape[:-1]
+    return x.new_empty(lead, dtype=torch.int64), x.new_empty(lead, dtype=torch.float32)

@@ -34,6 +34,8 @@ def test_ops_are_registered_with_shape_only_implementations():
         y, r = torch.ops.mdx.add_rms_norm(x, x, w, 1e-6)
         assert y.shape == x.shape and r.shape == x.shape
         assert torch.ops.mdx.silu_and_mul(x).shape == (2, 32, 128)
+        x0, p = torch.ops.mdx.lm_head_confidence(x, torch.empty(1000, 256, **bf), None)
+        assert x0.shape == (2, 32) and x0.dtype == torch.int64 and p.shape == (2, 32) and p.dtype == torch.float32
 
 
 def test_mutated_arguments_are_declared():
@@ -72,7 +74,8 @@ def test_traced_function_matches_direct_calls(dev):
         y = mod.rms_norm(mod.silu_and_mul(torch.cat([y, r], -1)), w, 1e-6)
         logits = torch.nn.functional.linear(y, head)
         x0, p, tr, cnt = mod.unmask_step(logits, tokens, 999, 0.9, 4, None)
-        return o, od, y, x0, p, tr, cnt
+        hx0, hp = mod.lm_head_confidence(y, head, None)           # hidden 512: a multiple of 128
+        return o, od, y, x0, p, tr, cnt, hx0, hp
 
     class Direct:
         store_kvcache = staticmethod(mdx.store_kvcache)
@@ -83,6 +86,7 @@ def test_traced_function_matches_direct_calls(dev):
         rms_norm = staticmethod(mdx.rms_norm)
         silu_and_mul = staticmethod(mdx.silu_and_mul)
         unmask_step = staticmethod(lambda lg, t, m, th, k_, tm: mdx.unmask_step(lg, t, m, th, k_, temperatures=tm))
+        lm_head_confidence = staticmethod(mdx.lm_head_confidence)
 
     def fresh():
         return (torch.zeros(2, 256, 2, 128, dtype=torch.bfloat16, device=dev), torch.zeros(2, 256, 2, 128, dtype=torch.bfloat16, device=dev),
