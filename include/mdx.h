@@ -138,8 +138,8 @@ int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void*
  * that is a multiple of Hkv, page_size % 32 == 0.  MDX_BF16 and MDX_F16 with d a multiple of 16 up to 128 run on the
  * 16-bit matrix instructions (narrower heads are padded with zeros on the way into LDS; the partials keep their
  * 128-wide layout).  MDX_F32, and 16-bit tensors whose d is another multiple of 4 up to 256 (flash-attn takes heads
- * of up to 256 columns), run in fp32 arithmetic on the fp32 matrix instruction: one workgroup per (sequence, KV head,
- * query tile) walks the whole context, no split and no workspace (the workspace query returns 0 for those widths; a
+ * of up to 256 columns), run in fp32 arithmetic on the fp32 matrix instruction: one workgroup per (sequence, query head,
+ * query tile) walks the whole context, no split over workgroups and no workspace (the workspace query returns 0 for those widths; a
  * workspace that is passed anyway is ignored); exact rather than fast.
  */
 int64_t mdx_paged_block_attn_workspace_bytes(int32_t bs, int32_t sq, int32_t num_q_heads,

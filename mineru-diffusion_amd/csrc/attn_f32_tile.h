@@ -48,8 +48,10 @@ __device__ __forceinline__ int row_of_reg(int i, int H) { return 8 * (i >> 2) + 
 // D: 128 or 256, the head width that registers and LDS are laid out for (narrower heads are padded with zeros;
 // products over the padding are skipped).
 template <int D> struct Lds {
-    static constexpr int kPitchK = D + 1;      // floats: the 32 keys of a fragment read (one column) fall into 32 banks
-    static constexpr int kPitchV = D + 4;      // rows stay 16-byte aligned; the two keys of a k-step fall into different banks
+    // floats; rows stay 16-byte aligned and consecutive rows shift by 4 banks: the 16-byte reads of 8 consecutive keys
+    // (K fragments: four columns of a key per read) cover all banks once, and so do the two keys of a V k-step
+    static constexpr int kPitchK = D + 4;
+    static constexpr int kPitchV = D + 4;
     static constexpr int kFloats = kTileKeys * (kPitchK + kPitchV);
     static constexpr int kBytes = kFloats * (int)sizeof(float);
     static __device__ __forceinline__ float* k_tile(float* lds) { return lds; }
@@ -73,8 +75,7 @@ template <typename T, int D>
 __device__ __forceinline__ void stage4(float* lds, int row, int c4, const T* k4, const T* v4) {
     f32x4 kx = f32x4{0.f, 0.f, 0.f, 0.f}, vx = kx;
     if (k4) { kx = load4(k4); vx = load4(v4); }
-    float* kd = Lds<D>::k_tile(lds) + row * Lds<D>::kPitchK + 4 * c4;
-    kd[0] = kx[0]; kd[1] = kx[1]; kd[2] = kx[2]; kd[3] = kx[3];
+    *reinterpret_cast<f32x4*>(Lds<D>::k_tile(lds) + row * Lds<D>::kPitchK + 4 * c4) = kx;
     *reinterpret_cast<f32x4*>(Lds<D>::v_tile(lds) + row * Lds<D>::kPitchV + 4 * c4) = vx;
 }
 
@@ -96,14 +97,19 @@ template <int D, typename Visible>
 __device__ __forceinline__ void tile_step(const float* lds, const float (&q)[D / 2], State<D>& st, float c, int width, int lane, Visible visible)
 {
     const int H = lane >> 5, r = lane & 31;
-    // ---- S^T = K Q^T: rows = keys, columns = queries; k-step j covers d = 2 j, 2 j + 1 ----
+    // ---- S^T = K Q^T: rows = keys, columns = queries; k-step j covers d = 2 j, 2 j + 1 (half-wavefront H holds d = 2 j + H);
+    //      a 16-byte read of key r's columns 4 m .. 4 m + 3 feeds the k-steps 2 m and 2 m + 1 ----
     f32x16 s;
 #pragma unroll
     for (int i = 0; i < 16; ++i) s[i] = 0.f;
-    const float* krow = Lds<D>::k_tile(const_cast<float*>(lds)) + r * Lds<D>::kPitchK + H;
+    const float* krow = Lds<D>::k_tile(const_cast<float*>(lds)) + r * Lds<D>::kPitchK;
 #pragma unroll
-    for (int j = 0; j < D / 2; ++j)
-        if (2 * j < width) s = __builtin_amdgcn_mfma_f32_32x32x2f32(krow[2 * j], q[j], s, 0, 0, 0);
+    for (int m = 0; m < D / 4; ++m) {
+        if (4 * m >= width) continue;
+        const f32x4 kx = *reinterpret_cast<const f32x4*>(krow + 4 * m);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(H ? kx[1] : kx[0], q[2 * m], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(H ? kx[3] : kx[2], q[2 * m + 1], s, 0, 0, 0);
+    }
 
     // ---- online softmax over the keys, base 2 ----
     float mx = kMinusBig;

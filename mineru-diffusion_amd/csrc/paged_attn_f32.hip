@@ -5,9 +5,10 @@
 // itself runs bf16 with d = 128, so this is the path for callers outside the model's own configuration.
 // Arithmetic and layout: attn_f32_tile.h.
 //
-// A workgroup of 4 wavefronts serves one (sequence, KV head, tile of 32 queries): it walks the sequence's
-// context once per round of four query heads of that KV head, a wavefront per head, all of them on the same
-// K / V tile in LDS.  No split over the keys and no workspace: every output row is written once, by its wavefront.
+// A workgroup serves one (sequence, query head, tile of 32 queries).  Its NW wavefronts (4 for heads of up to 128
+// columns, 2 for wider ones: what fits in LDS) take consecutive tiles of 32 keys, NW tiles staged at a time, each
+// wavefront with its own running softmax state; at the end the states are merged through LDS and every wavefront
+// writes its share of the head's columns.  No split over workgroups and no workspace.
 // The semantics are those of the 16-bit kernel: non-causal, the first min(context_lens[b], max_pages x
 // page_size) keys through block_table[b]; keys on a page id outside [0, num_pages) are left out; a sequence
 // without any key yields zeros.
@@ -17,9 +18,6 @@
 namespace {
 
 using namespace mdx_attn_f32;
-
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / 64;
 
 struct PagedWideParams {
     const void* q; void* o; const void* k_cache; const void* v_cache;
@@ -32,14 +30,17 @@ struct PagedWideParams {
     float c;                                        // scale * log2(e)
 };
 
-template <typename T, int D>
-__global__ __launch_bounds__(kThreads, 1) void paged_attn_f32_kernel(const PagedWideParams P)
+template <typename T, int D, int NW>
+__global__ __launch_bounds__(64 * NW, 1) void paged_attn_f32_kernel(const PagedWideParams P)
 {
-    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int kThreads = 64 * NW;
+    constexpr int kTileFloats = Lds<D>::kFloats;
+    extern __shared__ __attribute__((aligned(16))) float lds[];          // NW tiles (K and V of 32 keys each)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int H = lane >> 5, r = lane & 31;
-    const int kvh = blockIdx.x, qt = blockIdx.y, b = blockIdx.z;
+    const int head = blockIdx.x, qt = blockIdx.y, b = blockIdx.z;
+    const int kvh = head / P.heads_per_kv;
     const int width = P.head_dim;
 
     const int64_t room = (int64_t)P.max_pages * P.page_size;
@@ -53,54 +54,98 @@ __global__ __launch_bounds__(kThreads, 1) void paged_attn_f32_kernel(const Paged
     const T* kc = static_cast<const T*>(P.k_cache) + (int64_t)kvh * P.c_sh;
     const T* vc = static_cast<const T*>(P.v_cache) + (int64_t)kvh * P.c_sh;
 
-    for (int h0 = 0; h0 < P.heads_per_kv; h0 += kWaves) {
-        const bool active = h0 + wave < P.heads_per_kv;       // uniform per wavefront
-        const int head = kvh * P.heads_per_kv + h0 + wave;
-        float q[D / 2];
-        load_q<T, D>(q, (active && row_ok) ? static_cast<const T*>(P.q) + (int64_t)b * P.q_sb + (int64_t)qrow * P.q_ss + (int64_t)head * P.q_sh : nullptr, H, width);
-        State<D> st;
-        st.init();
-        for (int t = 0; t < n_tiles; ++t) {
-            const int key0 = t * kTileKeys;
-            // a tile never straddles a page (page_size % 32 == 0): one look-up, uniform
-            const int64_t page = bt[key0 / P.page_size];
-            const bool page_ok = page >= 0 && page < P.num_pages;
-            __syncthreads();                                   // the previous tile has been read by everybody
-            if (page_ok) {
-                const int64_t base = page * P.c_sp + (int64_t)(key0 % P.page_size) * P.c_st;
+    float q[D / 2];
+    load_q<T, D>(q, row_ok ? static_cast<const T*>(P.q) + (int64_t)b * P.q_sb + (int64_t)qrow * P.q_ss + (int64_t)head * P.q_sh : nullptr, H, width);
+    State<D> st;
+    st.init();
+    for (int t0 = 0; t0 < n_tiles; t0 += NW) {
+        __syncthreads();                                       // the previous tiles have been read by everybody
+        // ---- tiles t0 .. t0 + NW - 1 into LDS, all threads on each (a tile never straddles a page: page_size % 32 == 0) ----
+        unsigned tile_ok = 0;                                  // bit i: tile t0 + i exists and lies on a valid page (uniform)
 #pragma unroll
-                for (int p = 0; p < kTileKeys * (D / 4) / kThreads; ++p) {
-                    const int u = tid + kThreads * p;
-                    const int row = u / (D / 4), c4 = u % (D / 4);
-                    const bool real = key0 + row < ctx && 4 * c4 < width;
-                    const int64_t off = base + (int64_t)row * P.c_st + 4 * c4;
-                    stage4<T, D>(lds, row, c4, real ? kc + off : nullptr, real ? vc + off : nullptr);
-                }
+        for (int i = 0; i < NW; ++i) {
+            const int key0 = (t0 + i) * kTileKeys;
+            if (key0 >= ctx) break;
+            const int64_t page = bt[key0 / P.page_size];
+            if (page < 0 || page >= P.num_pages) continue;
+            tile_ok |= 1u << i;
+            const int64_t base = page * P.c_sp + (int64_t)(key0 % P.page_size) * P.c_st;
+#pragma unroll
+            for (int p = 0; p < kTileKeys * (D / 4) / kThreads; ++p) {
+                const int u = tid + kThreads * p;
+                const int row = u / (D / 4), c4 = u % (D / 4);
+                const bool real = key0 + row < ctx && 4 * c4 < width;
+                const int64_t off = base + (int64_t)row * P.c_st + 4 * c4;
+                stage4<T, D>(lds + i * kTileFloats, row, c4, real ? kc + off : nullptr, real ? vc + off : nullptr);
             }
-            __syncthreads();
-            if (page_ok && active)
-                tile_step<D>(lds, q, st, P.c, width, lane, [&](int key) { return key0 + key < ctx; });
         }
-        if (active)
-            store_o<T, D>(row_ok ? static_cast<T*>(P.o) + (int64_t)b * P.o_sb + (int64_t)qrow * P.o_ss + (int64_t)head * P.o_sh : nullptr, st, H, width);
+        __syncthreads();
+        if ((tile_ok >> wave) & 1u) {
+            const int key0 = (t0 + wave) * kTileKeys;
+            tile_step<D>(lds + wave * kTileFloats, q, st, P.c, width, lane, [&](int key) { return key0 + key < ctx; });
+        }
+    }
+
+    // ---- merge the NW states through LDS: every wavefront folds, and stores, the column tiles dt = wave, wave + NW, ... ----
+    constexpr int kStateFloats = (D / 32) * 16 * 64 + 2 * 64;                  // O as [dt][register][lane], then m, l
+    static_assert(NW * kStateFloats <= NW * kTileFloats, "merge buffer exceeds the tile region");
+    st.l += __shfl_xor(st.l, 32);                                              // a state is now (m, l, O) per query
+    __syncthreads();                                                           // the last tiles have been read by everybody
+    {
+        float* dst = lds + wave * kStateFloats;
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[(dt * 16 + i) * 64 + lane] = st.o[dt][i];
+        dst[(D / 32) * 16 * 64 + lane] = st.m;
+        dst[(D / 32) * 16 * 64 + 64 + lane] = st.l;
+    }
+    __syncthreads();
+    float w[NW];
+    float M = kMinusBig, l_all = 0.f;
+#pragma unroll
+    for (int s = 0; s < NW; ++s) { w[s] = lds[s * kStateFloats + (D / 32) * 16 * 64 + lane]; M = fmaxf(M, w[s]); }
+#pragma unroll
+    for (int s = 0; s < NW; ++s) {
+        w[s] = __builtin_amdgcn_exp2f(w[s] - M);
+        l_all += lds[s * kStateFloats + (D / 32) * 16 * 64 + 64 + lane] * w[s];
+    }
+    if (!row_ok) return;
+    const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;                        // no key at all: zeros
+    T* orow = static_cast<T*>(P.o) + (int64_t)b * P.o_sb + (int64_t)qrow * P.o_ss + (int64_t)head * P.o_sh;
+#pragma unroll
+    for (int dt = 0; dt < D / 32; ++dt) {
+        if (dt % NW != wave || dt * 32 >= width) continue;                     // (uniform per wavefront)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NW; ++s)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += lds[s * kStateFloats + (dt * 16 + 4 * g + e) * 64 + lane] * w[s];
+            const int d = dt * 32 + 8 * g + 4 * H;
+            if (d < width) store4(orow + d, f32x4{acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv});
+        }
     }
 }
 
 template <typename T, int D>
-int launch(const PagedWideParams& P, int bs, int num_kv_heads, hipStream_t stream)
+int launch(const PagedWideParams& P, int bs, int num_q_heads, hipStream_t stream)
 {
+    constexpr int NW = D <= 128 ? 4 : 2;            // tiles of 32 keys that fit in LDS side by side
+    constexpr int kLdsBytes = NW * Lds<D>::kBytes;
     // the kernel's LDS limit is raised once per device
     static std::atomic<bool> raised[64];
     int device = 0;
     hipError_t e = hipGetDevice(&device);
     MDX_REQUIRE(e == hipSuccess && device >= 0 && device < 64, MDX_ELAUNCH, "paged_block_attn: no current device (%s)", hipGetErrorString(e));
     if (!raised[device].load(std::memory_order_acquire)) {
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(paged_attn_f32_kernel<T, D>), hipFuncAttributeMaxDynamicSharedMemorySize, Lds<D>::kBytes);
-        MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "paged_block_attn: cannot reserve %d bytes of LDS (%s)", Lds<D>::kBytes, hipGetErrorString(e));
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(paged_attn_f32_kernel<T, D, NW>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        MDX_REQUIRE(e == hipSuccess, MDX_ELAUNCH, "paged_block_attn: cannot reserve %d bytes of LDS (%s)", kLdsBytes, hipGetErrorString(e));
         raised[device].store(true, std::memory_order_release);
     }
-    const dim3 grid((unsigned)num_kv_heads, (unsigned)((P.sq + 31) / 32), (unsigned)bs);
-    paged_attn_f32_kernel<T, D><<<grid, kThreads, Lds<D>::kBytes, stream>>>(P);
+    const dim3 grid((unsigned)num_q_heads, (unsigned)((P.sq + 31) / 32), (unsigned)bs);
+    paged_attn_f32_kernel<T, D, NW><<<grid, 64 * NW, kLdsBytes, stream>>>(P);
     return mdx::check_launch("paged_block_attn (fp32 arithmetic)");
 }
 
@@ -127,7 +172,7 @@ int launch_paged_f32(const void* q, void* o, const void* k_cache, const void* v_
                 o_stride_b % 4 == 0 && o_stride_s % 4 == 0 && o_stride_h % 4 == 0 &&
                 cache_stride_page % 4 == 0 && cache_stride_tok % 4 == 0 && cache_stride_head % 4 == 0,
                 MDX_EUNSUPPORTED, "paged_block_attn: tensors must be aligned to four elements with strides that are multiples of 4 elements");
-    MDX_REQUIRE(bs <= 65535 && num_kv_heads <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: fp32 arithmetic takes up to 65535 sequences");
+    MDX_REQUIRE(bs <= 65535 && num_q_heads <= 65535, MDX_EUNSUPPORTED, "paged_block_attn: fp32 arithmetic takes up to 65535 sequences");
     PagedWideParams P;
     P.q = q; P.o = o; P.k_cache = k_cache; P.v_cache = v_cache;
     P.q_sb = q_stride_b; P.q_ss = q_stride_s; P.q_sh = q_stride_h;
@@ -139,9 +184,9 @@ int launch_paged_f32(const void* q, void* o, const void* k_cache, const void* v_
     P.c = scale * kLog2e;
     const bool wide = head_dim > 128;
     switch (dtype) {
-    case MDX_F32:  return wide ? launch<float, 256>(P, bs, num_kv_heads, stream) : launch<float, 128>(P, bs, num_kv_heads, stream);
-    case MDX_F16:  return wide ? launch<_Float16, 256>(P, bs, num_kv_heads, stream) : launch<_Float16, 128>(P, bs, num_kv_heads, stream);
-    case MDX_BF16: return wide ? launch<__bf16, 256>(P, bs, num_kv_heads, stream) : launch<__bf16, 128>(P, bs, num_kv_heads, stream);
+    case MDX_F32:  return wide ? launch<float, 256>(P, bs, num_q_heads, stream) : launch<float, 128>(P, bs, num_q_heads, stream);
+    case MDX_F16:  return wide ? launch<_Float16, 256>(P, bs, num_q_heads, stream) : launch<_Float16, 128>(P, bs, num_q_heads, stream);
+    case MDX_BF16: return wide ? launch<__bf16, 256>(P, bs, num_q_heads, stream) : launch<__bf16, 128>(P, bs, num_q_heads, stream);
     }
     return mdx::fail(MDX_EUNSUPPORTED, "paged_block_attn: dtype %d", dtype);
 }
