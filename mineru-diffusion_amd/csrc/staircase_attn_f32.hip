@@ -30,7 +30,7 @@ struct WideParams {
 
 // T: element type of q/k/v/o.  D: 128 or 256, the head width that registers and LDS are laid out for.
 template <typename T, int D>
-__global__ __launch_bounds__(kThreads, 1) void staircase_attn_f32_kernel(const WideParams P)
+__global__ __launch_bounds__(kThreads, D <= 128 ? 2 : 1) void staircase_attn_f32_kernel(const WideParams P)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
 
