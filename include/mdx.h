@@ -100,7 +100,7 @@ int mdx_store_kvcache(const void* key, const void* value,
  * strides that are multiples of 8 elements, o's of 4).  MDX_F32, and 16-bit
  * tensors whose d is another multiple of 4 up to 256, run in fp32 arithmetic
  * on the fp32 matrix instruction (probabilities never rounded, 16-bit inputs
- * widened; exact rather than fast: about a fifteenth of the 16-bit kernels' rate;
+ * widened; exact rather than fast: about a tenth of the 16-bit kernels' rate;
  * tensors aligned to four elements with strides that are multiples of 4).
  */
 int mdx_staircase_attn_varlen(const void* q, const void* k, const void* v, void* o,
